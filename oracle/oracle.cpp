@@ -1,0 +1,674 @@
+// TEST INFRASTRUCTURE ONLY -- see oracle.h.  CPU restatement of the arithmetic of the reference's
+// inference path (llama_cu.cu kernels 30-540, forward pass 1073-1210, quantiser transform.cu:28-87).
+// fp16 is storage only: every value is widened to fp32, combined in fp32 and rounded back to fp16
+// (round-to-nearest-even) exactly where the reference stores a __half.
+#include "oracle.h"
+
+#include <immintrin.h>
+#include <math.h>
+#include <omp.h>
+#include <stdlib.h>
+#include <string.h>
+
+#include <vector>
+
+namespace {
+
+inline float h2f(uint16_t h) { return _cvtsh_ss(h); }
+inline uint16_t f2h(float f) { return _cvtss_sh(f, _MM_FROUND_TO_NEAREST_INT | _MM_FROUND_NO_EXC); }
+
+inline uint64_t splitmix64(uint64_t z) {
+  z += 0x9E3779B97F4A7C15ull;
+  z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+  z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+  return z ^ (z >> 31);
+}
+
+inline int sum16(uint64_t h) {
+  return int(h & 0xFFFF) + int((h >> 16) & 0xFFFF) + int((h >> 32) & 0xFFFF) + int(h >> 48);
+}
+
+// Lane-0 value of a CUDA xor-shuffle all-reduce over `n` slots (n a power of two): at every level
+// slot t takes v[t] op v[t ^ off]; floating-point + and max are commutative, so all slots agree
+// and the value is this pairwise tree.
+template <typename Op>
+inline float butterfly(float* v, int n, Op op) {
+  for (int off = n / 2; off > 0; off /= 2) {
+    for (int t = 0; t < off; ++t) {
+      v[t] = op(v[t], v[t + off]);
+    }
+  }
+  return v[0];
+}
+
+// The block reduction used by rms_norm (llama_cu.cu:75-100) and softmax_rows (442-493):
+// 256 threads hold one partial each, 8 warps of 32 reduce by xor shuffles 16..1, then the
+// 8 warp results reduce by xor shuffles 4..1.
+template <typename Op>
+inline float block_reduce_256(float* part, Op op) {
+  float warp[8];
+  for (int w = 0; w < 8; ++w) {
+    warp[w] = butterfly(part + 32 * w, 32, op);
+  }
+  return butterfly(warp, 8, op);
+}
+
+inline float addf(float a, float b) { return a + b; }
+inline float maxf(float a, float b) { return fmaxf(a, b); }
+
+inline void row_to_float(float* dst, const uint16_t* src, int K) {
+  int k = 0;
+  for (; k + 8 <= K; k += 8) {
+    _mm256_storeu_ps(dst + k, _mm256_cvtph_ps(_mm_loadu_si128((const __m128i*)(src + k))));
+  }
+  for (; k < K; ++k) {
+    dst[k] = h2f(src[k]);
+  }
+}
+
+// dequantize_absmax_one, llama_cu.cu:287-289: fp32 product rounded once to fp16.
+inline uint16_t dequant_one(uint8_t q, uint16_t scale) { return f2h((float(q) - 127.5f) * h2f(scale)); }
+
+inline void row_u8_to_float(float* dst, const uint8_t* codes, const uint16_t* scales, int K, int block) {
+  for (int k = 0; k < K; ++k) {
+    dst[k] = h2f(dequant_one(codes[k], scales[k / block]));
+  }
+}
+
+// 16 interleaved partial sums (k mod 16), combined 8,4,2,1.
+inline float dot16(const float* x, const float* w, int K) {
+  __m256 a0 = _mm256_setzero_ps(), a1 = _mm256_setzero_ps();
+  int k = 0;
+  for (; k + 16 <= K; k += 16) {
+    a0 = _mm256_fmadd_ps(_mm256_loadu_ps(x + k), _mm256_loadu_ps(w + k), a0);
+    a1 = _mm256_fmadd_ps(_mm256_loadu_ps(x + k + 8), _mm256_loadu_ps(w + k + 8), a1);
+  }
+  float acc[16];
+  _mm256_storeu_ps(acc, a0);
+  _mm256_storeu_ps(acc + 8, a1);
+  for (; k < K; ++k) {
+    acc[k % 16] = fmaf(x[k], w[k], acc[k % 16]);
+  }
+  return butterfly(acc, 16, addf);
+}
+
+// four rows of x against one row of w; same summation order as dot16
+inline void dot16x4(const float* x0, const float* x1, const float* x2, const float* x3, const float* w,
+                    int K, float* out) {
+  __m256 a[4][2];
+  for (int i = 0; i < 4; ++i) {
+    a[i][0] = _mm256_setzero_ps();
+    a[i][1] = _mm256_setzero_ps();
+  }
+  const float* xs[4] = {x0, x1, x2, x3};
+  int k = 0;
+  for (; k + 16 <= K; k += 16) {
+    __m256 w0 = _mm256_loadu_ps(w + k), w1 = _mm256_loadu_ps(w + k + 8);
+    for (int i = 0; i < 4; ++i) {
+      a[i][0] = _mm256_fmadd_ps(_mm256_loadu_ps(xs[i] + k), w0, a[i][0]);
+      a[i][1] = _mm256_fmadd_ps(_mm256_loadu_ps(xs[i] + k + 8), w1, a[i][1]);
+    }
+  }
+  for (int i = 0; i < 4; ++i) {
+    float acc[16];
+    _mm256_storeu_ps(acc, a[i][0]);
+    _mm256_storeu_ps(acc + 8, a[i][1]);
+    for (int kk = k; kk < K; ++kk) {
+      acc[kk % 16] = fmaf(xs[i][kk], w[kk], acc[kk % 16]);
+    }
+    out[i] = butterfly(acc, 16, addf);
+  }
+}
+
+inline uint16_t epilogue(float acc, float beta, uint16_t old) {
+  // llama_cu.cu:120, 213, 279, 360: acc + beta * old, one rounding to fp16.  beta == 0 skips the
+  // read of the old value (the reference multiplies it by zero; its buffers start zeroed).
+  if (beta == 0.0f) {
+    return f2h(acc);
+  }
+  return f2h(fmaf(beta, h2f(old), acc));
+}
+
+void matmul_tiled(uint16_t* out, const uint16_t* lhs, const uint16_t* rhs_h, const uint8_t* rhs_q,
+                  const uint16_t* scales, int M, int K, int N, int block, float beta) {
+  std::vector<float> xf((size_t)M * K);
+#pragma omp parallel for schedule(static)
+  for (int m = 0; m < M; ++m) {
+    row_to_float(&xf[(size_t)m * K], lhs + (size_t)m * K, K);
+  }
+#pragma omp parallel
+  {
+    std::vector<float> wf(K);
+#pragma omp for schedule(static)
+    for (int n = 0; n < N; ++n) {
+      if (rhs_q) {
+        row_u8_to_float(wf.data(), rhs_q + (size_t)n * K, scales + (size_t)n * (K / block), K, block);
+      } else {
+        row_to_float(wf.data(), rhs_h + (size_t)n * K, K);
+      }
+      int m = 0;
+      for (; m + 4 <= M; m += 4) {
+        float r[4];
+        const float* x = &xf[(size_t)m * K];
+        dot16x4(x, x + K, x + 2 * (size_t)K, x + 3 * (size_t)K, wf.data(), K, r);
+        for (int i = 0; i < 4; ++i) {
+          size_t o = (size_t)(m + i) * N + n;
+          out[o] = epilogue(r[i], beta, out[o]);
+        }
+      }
+      for (; m < M; ++m) {
+        size_t o = (size_t)m * N + n;
+        out[o] = epilogue(dot16(&xf[(size_t)m * K], wf.data(), K), beta, out[o]);
+      }
+    }
+  }
+}
+
+}  // namespace
+
+extern "C" {
+
+int orc_num_threads(void) { return omp_get_max_threads(); }
+
+void orc_fill_normal_f16(uint16_t* out, size_t n, uint64_t seed, uint64_t stream, float std) {
+  const uint64_t key = splitmix64(seed ^ (stream * 0xD1B54A32D192ED03ull));
+  const double sigma = sqrt(8.0 * (65536.0 * 65536.0 - 1.0) / 12.0);
+  const float scale = (float)((double)std / sigma);
+#pragma omp parallel for schedule(static)
+  for (size_t i = 0; i < n; ++i) {
+    uint64_t h1 = splitmix64(key + i);
+    uint64_t h2 = splitmix64(h1);
+    int s = sum16(h1) + sum16(h2) - 262140;
+    out[i] = f2h((float)s * scale);
+  }
+}
+
+// transform.cu:28-72.  absmax in fp32 (max is exact in any order), scale = fp16(absmax / 127.5f),
+// code = (uint8) roundf(127.5f + x / scale) with IEEE division and round-half-away.  The cast is
+// defined here as saturating with NaN -> 0 (what the GPU conversion does); in-range inputs never
+// reach that.
+void orc_quantize_absmax_u8(uint8_t* codes, uint16_t* scales, const uint16_t* in, size_t rows,
+                            size_t cols, int block) {
+  const size_t nblk = cols / block;
+#pragma omp parallel for schedule(static)
+  for (size_t r = 0; r < rows; ++r) {
+    for (size_t b = 0; b < nblk; ++b) {
+      const uint16_t* src = in + r * cols + b * block;
+      float absmax = 0.0f;
+      for (int i = 0; i < block; ++i) {
+        absmax = fmaxf(absmax, fabsf(h2f(src[i])));
+      }
+      const uint16_t sh = f2h(absmax / 127.5f);
+      scales[r * nblk + b] = sh;
+      const float s = h2f(sh);
+      uint8_t* dst = codes + r * cols + b * block;
+      for (int i = 0; i < block; ++i) {
+        float v = roundf(127.5f + h2f(src[i]) / s);
+        dst[i] = (v >= 255.0f) ? 255 : (v > 0.0f ? (uint8_t)v : 0);
+      }
+    }
+  }
+}
+
+// transform.cu:74-87
+void orc_dequantize_absmax_u8(uint16_t* out, const uint16_t* scales, const uint8_t* codes,
+                              size_t rows, size_t cols, int block) {
+  const size_t nblk = cols / block;
+#pragma omp parallel for schedule(static)
+  for (size_t r = 0; r < rows; ++r) {
+    for (size_t c = 0; c < cols; ++c) {
+      out[r * cols + c] = f2h((float(codes[r * cols + c]) - 127.5f) * h2f(scales[r * nblk + c / block]));
+    }
+  }
+}
+
+void orc_matmul_nt(uint16_t* out, const uint16_t* lhs, const uint16_t* rhs, int M, int K, int N,
+                   float beta, int flavour) {
+  if (flavour == 0) {
+    // llama_cu.cu:111-122
+#pragma omp parallel for schedule(static)
+    for (int c = 0; c < N; ++c) {
+      for (int r = 0; r < M; ++r) {
+        float sum = 0;
+        for (int i = 0; i < K; ++i) {
+          sum += h2f(lhs[(size_t)r * K + i]) * h2f(rhs[(size_t)c * K + i]);  // product exact in fp32
+        }
+        size_t o = (size_t)r * N + c;
+        out[o] = epilogue(sum, beta, out[o]);
+      }
+    }
+    return;
+  }
+  matmul_tiled(out, lhs, rhs, nullptr, nullptr, M, K, N, 1, beta);
+}
+
+void orc_matmul_nt_u8(uint16_t* out, const uint16_t* lhs, const uint8_t* codes,
+                      const uint16_t* scales, int M, int K, int N, int block, float beta,
+                      int flavour) {
+  if (flavour == 0) {
+    // llama_cu.cu:125-145.  The literal 127.5 there is a double, so each term is formed in
+    // double and the running sum is rounded back to float after every addition.
+    const int nblk = K / block;
+#pragma omp parallel for schedule(static)
+    for (int c = 0; c < N; ++c) {
+      for (int r = 0; r < M; ++r) {
+        float sum = 0;
+        for (int i = 0; i < K; ++i) {
+          double term = (double)h2f(lhs[(size_t)r * K + i]) *
+                        ((double)float(codes[(size_t)c * K + i]) - 127.5) *
+                        (double)h2f(scales[(size_t)c * nblk + i / block]);
+          sum = (float)((double)sum + term);
+        }
+        size_t o = (size_t)r * N + c;
+        out[o] = epilogue(sum, beta, out[o]);
+      }
+    }
+    return;
+  }
+  matmul_tiled(out, lhs, nullptr, codes, scales, M, K, N, block, beta);
+}
+
+// llama_cu.cu:66-107.  rsqrt is restated as 1/sqrt with IEEE operations.
+void orc_rms_norm(uint16_t* out, const uint16_t* in, const uint16_t* weights, int rows, int cols,
+                  float eps) {
+#pragma omp parallel for schedule(static)
+  for (int row = 0; row < rows; ++row) {
+    const uint16_t* x = in + (size_t)row * cols;
+    float part[256];
+    for (int t = 0; t < 256; ++t) {
+      float s = 0.0f;
+      for (int i = t; i < cols; i += 256) {
+        float v = h2f(x[i]);
+        s += v * v;  // exact product
+      }
+      part[t] = s;
+    }
+    float sum = block_reduce_256(part, addf);
+    float rms_inv = 1.0f / sqrtf((sum / cols) + eps);
+    for (int i = 0; i < cols; ++i) {
+      uint16_t inner = f2h(h2f(x[i]) * rms_inv);
+      out[(size_t)row * cols + i] = f2h(h2f(weights[i]) * h2f(inner));  // __hmul: RN of exact product
+    }
+  }
+}
+
+// One interleaved pair, llama_cu.cu:381-387.  The two products-and-sum are restated with one
+// fused multiply-add each, which is how the expression contracts when compiled for a GPU.
+static inline void rotate_pair(uint16_t* o0, uint16_t* o1, uint16_t i0, uint16_t i1, float c, float s) {
+  float real = h2f(i0), imag = h2f(i1);
+  *o0 = f2h(fmaf(real, c, -(imag * s)));
+  *o1 = f2h(fmaf(real, s, imag * c));
+}
+
+static inline void rope_angle(int pos, int head_c, int head_dim, float theta, float* c, float* s) {
+  float angle = (float)pos / powf(theta, float(head_c) / head_dim);
+  *c = cosf(angle);
+  *s = sinf(angle);
+}
+
+void orc_rotary(uint16_t* out, const uint16_t* in, int rows, int cols, int n_heads, int pos_offset,
+                float theta) {
+  const int head_dim = cols / n_heads;
+#pragma omp parallel for schedule(static)
+  for (int r = 0; r < rows; ++r) {
+    for (int c = 0; c < cols; c += 2) {
+      float a_cos, a_sin;
+      rope_angle(pos_offset + r, c % head_dim, head_dim, theta, &a_cos, &a_sin);
+      size_t o = (size_t)r * cols + c;
+      rotate_pair(&out[o], &out[o + 1], in[o], in[o + 1], a_cos, a_sin);
+    }
+  }
+}
+
+// llama_cu.cu:400-428.  Rows of the output have stride T (the reference's writer uses n_new,
+// its readers T; the two agree in every call the forward pass makes).
+void orc_matmul_qk(uint16_t* out, const uint16_t* q, const uint16_t* k, int n_new, int T, int dim,
+                   int n_heads, int start_pos) {
+  const int head_dim = dim / n_heads;
+  const float denom = sqrtf(float(head_dim));
+#pragma omp parallel for collapse(2) schedule(static)
+  for (int head = 0; head < n_heads; ++head) {
+    for (int r = 0; r < n_new; ++r) {
+      for (int c = 0; c < T; ++c) {
+        size_t o = ((size_t)head * n_new + r) * T + c;
+        if (c > r + start_pos) {
+          out[o] = 0xFC00;  // -inf
+        } else {
+          float sum = 0;
+          for (int i = 0; i < head_dim; ++i) {
+            sum += h2f(q[(size_t)r * dim + head * head_dim + i]) * h2f(k[(size_t)c * dim + head * head_dim + i]);
+          }
+          out[o] = f2h(sum / denom);
+        }
+      }
+    }
+  }
+}
+
+// llama_cu.cu:433-499
+void orc_softmax_rows(uint16_t* out, const uint16_t* in, int rows, int w, float temp) {
+#pragma omp parallel for schedule(static)
+  for (int row = 0; row < rows; ++row) {
+    const uint16_t* x = in + (size_t)row * w;
+    uint16_t* y = out + (size_t)row * w;
+    float part[256];
+    for (int t = 0; t < 256; ++t) {
+      float m = -INFINITY;
+      for (int i = t; i < w; i += 256) {
+        m = fmaxf(m, h2f(x[i]) / temp);
+      }
+      part[t] = m;
+    }
+    const float max_val = block_reduce_256(part, maxf);
+    for (int t = 0; t < 256; ++t) {
+      float s = 0.0f;
+      for (int i = t; i < w; i += 256) {
+        s += expf(h2f(x[i]) / temp - max_val);
+      }
+      part[t] = s;
+    }
+    const float sum_exp = block_reduce_256(part, addf);
+    for (int i = 0; i < w; ++i) {
+      y[i] = f2h(expf(h2f(x[i]) / temp - max_val) / sum_exp);
+    }
+  }
+}
+
+// llama_cu.cu:511-531
+void orc_matmul_qkv(uint16_t* out, const uint16_t* p, const uint16_t* v, int n_new, int T, int dim,
+                    int n_heads) {
+  const int head_dim = dim / n_heads;
+#pragma omp parallel for collapse(2) schedule(static)
+  for (int r = 0; r < n_new; ++r) {
+    for (int head = 0; head < n_heads; ++head) {
+      float sum[512];
+      for (int j = 0; j < head_dim; ++j) sum[j] = 0.0f;
+      const uint16_t* prow = p + ((size_t)head * n_new + r) * T;
+      for (int i = 0; i < T; ++i) {  // i ascending for every output, as in the reference
+        float pv = h2f(prow[i]);
+        const uint16_t* vrow = v + (size_t)i * dim + head * head_dim;
+        for (int j = 0; j < head_dim; ++j) {
+          sum[j] += pv * h2f(vrow[j]);
+        }
+      }
+      for (int j = 0; j < head_dim; ++j) {
+        out[(size_t)r * dim + head * head_dim + j] = f2h(sum[j]);
+      }
+    }
+  }
+}
+
+// llama_cu.cu:533-539
+void orc_silu_mul(uint16_t* out, const uint16_t* a, const uint16_t* b, size_t size) {
+#pragma omp parallel for schedule(static)
+  for (size_t i = 0; i < size; ++i) {
+    float val = h2f(a[i]);
+    out[i] = f2h(val / (1.0f + expf(-val)) * h2f(b[i]));
+  }
+}
+
+void orc_embed(uint16_t* out, const int16_t* ids, int n_ids, int dim, const uint16_t* table) {
+  for (int t = 0; t < n_ids; ++t) {
+    memcpy(out + (size_t)t * dim, table + (size_t)ids[t] * dim, (size_t)dim * 2);
+  }
+}
+
+void orc_embed_u8(uint16_t* out, const int16_t* ids, int n_ids, int dim, const uint8_t* table,
+                  const uint16_t* scales, int block) {
+  const int nblk = dim / block;
+  for (int t = 0; t < n_ids; ++t) {
+    int id = ids[t];
+    for (int i = 0; i < dim; ++i) {
+      out[(size_t)t * dim + i] =
+          f2h((float(table[(size_t)id * dim + i]) - 127.5f) * h2f(scales[(size_t)id * nblk + i / block]));
+    }
+  }
+}
+
+int orc_argmax_first(const uint16_t* probs, int n) {
+  int best = 0;
+  for (int i = 1; i < n; ++i) {
+    if (h2f(probs[best]) < h2f(probs[i])) {
+      best = i;
+    }
+  }
+  return best;
+}
+
+// ------------------------------------------------------------------------------------------
+// whole model
+// ------------------------------------------------------------------------------------------
+struct orc_tensor {
+  std::vector<uint16_t> h;  // fp16 weights, or scales when quantised
+  std::vector<uint8_t> q;
+  int rows = 0, cols = 0;
+  bool quantised = false;
+};
+
+struct orc_model {
+  int dim, multiple_of, n_heads, n_layers, n_vocab, q_type, qblock, ffn;
+  float norm_eps;
+  orc_tensor tok_embeddings, output;
+  std::vector<uint16_t> norm;
+  struct layer {
+    orc_tensor wq, wk, wv, wo, w1, w2, w3;
+    std::vector<uint16_t> attn_norm, ffn_norm;
+  };
+  std::vector<layer> layers;
+};
+
+static void make_tensor(orc_model* m, orc_tensor& t, int rows, int cols, uint64_t seed, uint64_t stream,
+                        float std) {
+  t.rows = rows;
+  t.cols = cols;
+  std::vector<uint16_t> w((size_t)rows * cols);
+  orc_fill_normal_f16(w.data(), w.size(), seed, stream, std);
+  if (m->q_type == 1) {
+    t.quantised = true;
+    t.q.resize(w.size());
+    t.h.resize((size_t)rows * (cols / m->qblock));
+    orc_quantize_absmax_u8(t.q.data(), t.h.data(), w.data(), rows, cols, m->qblock);
+  } else {
+    t.h.swap(w);
+  }
+}
+
+orc_model* orc_model_create(int dim, int multiple_of, int n_heads, int n_layers, int n_vocab,
+                            float norm_eps, int q_type, int qblock, uint64_t seed,
+                            float weight_std) {
+  orc_model* m = new orc_model();
+  m->dim = dim;
+  m->multiple_of = multiple_of;
+  m->n_heads = n_heads;
+  m->n_layers = n_layers;
+  m->n_vocab = n_vocab;
+  m->norm_eps = norm_eps;
+  m->q_type = q_type;
+  m->qblock = qblock;
+  // llama_cu.cu:765-767
+  uint32_t hidden = (uint32_t)dim * 8 / 3;
+  m->ffn = (int)(((hidden + multiple_of - 1) / multiple_of) * multiple_of);
+  const uint16_t one = 0x3C00;
+  make_tensor(m, m->tok_embeddings, n_vocab, dim, seed, 1, weight_std);
+  make_tensor(m, m->output, n_vocab, dim, seed, 2, weight_std);
+  m->norm.assign(dim, one);
+  m->layers.resize(n_layers);
+  for (int l = 0; l < n_layers; ++l) {
+    auto& L = m->layers[l];
+    uint64_t base = 16 + 16 * (uint64_t)l;
+    make_tensor(m, L.wq, dim, dim, seed, base + 0, weight_std);
+    make_tensor(m, L.wk, dim, dim, seed, base + 1, weight_std);
+    make_tensor(m, L.wv, dim, dim, seed, base + 2, weight_std);
+    make_tensor(m, L.wo, dim, dim, seed, base + 3, weight_std);
+    make_tensor(m, L.w1, m->ffn, dim, seed, base + 4, weight_std);
+    make_tensor(m, L.w2, dim, m->ffn, seed, base + 5, weight_std);
+    make_tensor(m, L.w3, m->ffn, dim, seed, base + 6, weight_std);
+    L.attn_norm.assign(dim, one);
+    L.ffn_norm.assign(dim, one);
+  }
+  return m;
+}
+
+void orc_model_destroy(orc_model* m) { delete m; }
+int orc_model_ffn_dim(const orc_model* m) { return m->ffn; }
+
+const void* orc_model_tensor(const orc_model* m, uint64_t stream, const uint16_t** scales) {
+  const orc_tensor* t = nullptr;
+  if (stream == 1) {
+    t = &m->tok_embeddings;
+  } else if (stream == 2) {
+    t = &m->output;
+  } else if (stream >= 16) {
+    size_t l = (stream - 16) / 16;
+    int which = (int)((stream - 16) % 16);
+    if (l < m->layers.size() && which < 7) {
+      const orc_model::layer& L = m->layers[l];
+      const orc_tensor* tab[7] = {&L.wq, &L.wk, &L.wv, &L.wo, &L.w1, &L.w2, &L.w3};
+      t = tab[which];
+    }
+  }
+  if (!t) return nullptr;
+  if (t->quantised) {
+    if (scales) *scales = t->h.data();
+    return t->q.data();
+  }
+  if (scales) *scales = nullptr;
+  return t->h.data();
+}
+
+struct orc_context {
+  orc_model* model;
+  int context_len, start_pos, flavour, literal_rope;
+  float temperature;
+  std::vector<std::vector<uint16_t>> k, v;  // per layer [context_len][dim]
+  std::vector<float> rope_cos, rope_sin;    // [context_len][head_dim / 2]
+};
+
+static void rope_rows(const orc_context* c, uint16_t* out, const uint16_t* in, int rows, int pos_offset) {
+  const int dim = c->model->dim, head_dim = dim / c->model->n_heads, half = head_dim / 2;
+#pragma omp parallel for schedule(static)
+  for (int r = 0; r < rows; ++r) {
+    const float* cs = &c->rope_cos[(size_t)(pos_offset + r) * half];
+    const float* sn = &c->rope_sin[(size_t)(pos_offset + r) * half];
+    for (int col = 0; col < dim; col += 2) {
+      int pair = (col % head_dim) / 2;
+      size_t o = (size_t)r * dim + col;
+      rotate_pair(&out[o], &out[o + 1], in[o], in[o + 1], cs[pair], sn[pair]);
+    }
+  }
+}
+
+static void mm(const orc_context* c, uint16_t* out, const uint16_t* lhs, const orc_tensor& w, int M, float beta) {
+  // llama_cu.cu:1498-1523
+  if (w.quantised) {
+    orc_matmul_nt_u8(out, lhs, w.q.data(), w.h.data(), M, w.cols, w.rows, c->model->qblock, beta, c->flavour);
+  } else {
+    orc_matmul_nt(out, lhs, w.h.data(), M, w.cols, w.rows, beta, c->flavour);
+  }
+}
+
+orc_context* orc_context_create(orc_model* m, int context_len, float temperature, int matmul_flavour,
+                                int literal_rope) {
+  orc_context* c = new orc_context();
+  c->model = m;
+  c->context_len = context_len;
+  c->temperature = temperature;
+  c->flavour = matmul_flavour;
+  c->literal_rope = literal_rope;
+  c->start_pos = 0;
+  c->k.resize(m->n_layers);
+  c->v.resize(m->n_layers);
+  for (int l = 0; l < m->n_layers; ++l) {
+    c->k[l].assign((size_t)context_len * m->dim, 0);
+    c->v[l].assign((size_t)context_len * m->dim, 0);
+  }
+  const int head_dim = m->dim / m->n_heads, half = head_dim / 2;
+  c->rope_cos.resize((size_t)context_len * half);
+  c->rope_sin.resize((size_t)context_len * half);
+  for (int pos = 0; pos < context_len; ++pos) {
+    for (int p = 0; p < half; ++p) {
+      // same expression as orc_rotary / llama_cu.cu:381-385, theta = 10000 (the kernel default)
+      rope_angle(pos, 2 * p, head_dim, 10000.0f, &c->rope_cos[(size_t)pos * half + p],
+                 &c->rope_sin[(size_t)pos * half + p]);
+    }
+  }
+  return c;
+}
+
+void orc_context_destroy(orc_context* c) { delete c; }
+
+void orc_context_clear(orc_context* c) {
+  // llama_cu.cu:1004-1049: fresh zeroed KV, position 0
+  for (auto& t : c->k) std::fill(t.begin(), t.end(), 0);
+  for (auto& t : c->v) std::fill(t.begin(), t.end(), 0);
+  c->start_pos = 0;
+}
+
+int orc_context_start_pos(const orc_context* c) { return c->start_pos; }
+
+void orc_context_kv(orc_context* c, int layer, uint16_t* k_rot, uint16_t* v, int T) {
+  const size_t n = (size_t)T * c->model->dim;
+  if (k_rot) {
+    if (c->literal_rope) {
+      rope_rows(c, k_rot, c->k[layer].data(), T, 0);
+    } else {
+      memcpy(k_rot, c->k[layer].data(), n * 2);
+    }
+  }
+  if (v) memcpy(v, c->v[layer].data(), n * 2);
+}
+
+int orc_context_next_token(orc_context* c, const int16_t* tokens, int n, uint16_t* hidden,
+                           uint16_t* logits_out, uint16_t* probs_out) {
+  orc_model* m = c->model;
+  const int dim = m->dim, ffn = m->ffn, H = m->n_heads;
+  const int sp = c->start_pos, T = sp + n;
+  if (T > c->context_len || n <= 0) return -1;  // llama_cu.cu:1074 asserts
+  std::vector<uint16_t> x((size_t)n * dim), norm((size_t)n * dim), xq((size_t)n * dim),
+      xk((size_t)T * dim), att((size_t)n * dim), w1((size_t)n * ffn), w3((size_t)n * ffn),
+      silu((size_t)n * ffn), qk((size_t)H * n * T);
+  // 1087-1097
+  if (m->tok_embeddings.quantised) {
+    orc_embed_u8(x.data(), tokens, n, dim, m->tok_embeddings.q.data(), m->tok_embeddings.h.data(), m->qblock);
+  } else {
+    orc_embed(x.data(), tokens, n, dim, m->tok_embeddings.h.data());
+  }
+  for (int l = 0; l < m->n_layers; ++l) {
+    auto& L = m->layers[l];
+    uint16_t* kc = c->k[l].data();
+    uint16_t* vc = c->v[l].data();
+    orc_rms_norm(norm.data(), x.data(), L.attn_norm.data(), n, dim, m->norm_eps);  // 1129
+    mm(c, xq.data(), norm.data(), L.wq, n, 0.0f);                                  // 1144
+    rope_rows(c, xq.data(), xq.data(), n, sp);                                     // 1146
+    mm(c, kc + (size_t)sp * dim, norm.data(), L.wk, n, 0.0f);                      // 1150
+    const uint16_t* krot;
+    if (c->literal_rope) {
+      rope_rows(c, xk.data(), kc, T, 0);                                           // 1152
+      krot = xk.data();
+    } else {
+      rope_rows(c, kc + (size_t)sp * dim, kc + (size_t)sp * dim, n, sp);
+      krot = kc;
+    }
+    mm(c, vc + (size_t)sp * dim, norm.data(), L.wv, n, 0.0f);                      // 1156
+    orc_matmul_qk(qk.data(), xq.data(), krot, n, T, dim, H, sp);                   // 1163
+    orc_softmax_rows(qk.data(), qk.data(), H * n, T, 1.0f);                        // 1166
+    orc_matmul_qkv(att.data(), qk.data(), vc, n, T, dim, H);                       // 1170
+    mm(c, x.data(), att.data(), L.wo, n, 1.0f);                                    // 1174
+    orc_rms_norm(norm.data(), x.data(), L.ffn_norm.data(), n, dim, m->norm_eps);   // 1176
+    mm(c, w1.data(), norm.data(), L.w1, n, 0.0f);                                  // 1180
+    mm(c, w3.data(), norm.data(), L.w3, n, 0.0f);                                  // 1181
+    orc_silu_mul(silu.data(), w1.data(), w3.data(), (size_t)n * ffn);              // 1183
+    mm(c, x.data(), silu.data(), L.w2, n, 1.0f);                                   // 1185
+  }
+  if (hidden) memcpy(hidden, x.data(), x.size() * 2);
+  orc_rms_norm(norm.data(), x.data(), m->norm.data(), n, dim, m->norm_eps);        // 1191
+  std::vector<uint16_t> logits(m->n_vocab);
+  mm(c, logits.data(), norm.data() + (size_t)(n - 1) * dim, m->output, 1, 0.0f);   // 1194-1195
+  if (logits_out) memcpy(logits_out, logits.data(), logits.size() * 2);
+  orc_softmax_rows(logits.data(), logits.data(), 1, m->n_vocab, c->temperature);   // 1196
+  if (probs_out) memcpy(probs_out, logits.data(), logits.size() * 2);
+  c->start_pos += n;                                                               // 1201
+  return orc_argmax_first(logits.data(), m->n_vocab);                              // 1205-1209
+}
+
+}  // extern "C"

@@ -1,0 +1,116 @@
+/*
+ * TEST INFRASTRUCTURE ONLY.  CPU restatement of the arithmetic of eiz/llama.cu's
+ * inference path.  Nothing that ships (the HIP library, the host model code, the
+ * command line tools) may include, link or call this file; only tests/, the smoke
+ * check and the cpu_baseline leg of bench.py do, and only as the checker.
+ *
+ * Every function cites the reference lines it restates (paths relative to the
+ * reference checkout).  fp16 values travel as uint16_t bit patterns.
+ *
+ * Parity status of each function (what pins it):
+ *   orc_quantize_absmax_u8 / orc_dequantize_absmax_u8 : IEEE-only arithmetic, pinned by the
+ *       hand-computed known-answer block, the exhaustive 65536-input sweep against numpy
+ *       float32/float16 and the absmax/code-range invariants (tests/test_oracle_quant.py).
+ *   orc_matmul_nt[_u8] : pinned by float64 brute force, identity / one-hot / beta special cases.
+ *   orc_rms_norm, orc_rotary, orc_softmax_rows, orc_silu_mul, orc_matmul_qk, orc_matmul_qkv,
+ *   orc_embed[_u8], orc_argmax_first : pinned by closed forms and float64 restatements written
+ *       independently in numpy (tests/test_oracle_ops.py).
+ *   orc_context_next_token : pinned by an independent numpy float64 forward pass on a tiny model
+ *       (tolerance) and by the prefill-then-decode == longer-prefill invariant.
+ * The reference holds no golden vectors for any of these (it has no tests), and its CUDA sources
+ * cannot be compiled here, so no oracle/_ref build exists.
+ */
+#ifndef LLAMA_ORACLE_H
+#define LLAMA_ORACLE_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ---- seeded synthetic tensors (not from the reference: the shared test-input recipe) ---- */
+/* value[i] = fp16_rn( float(S - 262140) * scale ), S = sum of the eight 16-bit fields of
+ * splitmix64(key + i) and splitmix64 of that, key = splitmix64(seed ^ stream * 0xD1B54A32D192ED03),
+ * scale = float(std / sqrt(8 * (65536^2 - 1) / 12)).  Integer-exact, so host and GPU agree bit for bit. */
+void orc_fill_normal_f16(uint16_t* out, size_t n, uint64_t seed, uint64_t stream, float std);
+
+/* ---- int8 absmax block quantiser: transform.cu:28-72 and 74-87 ---- */
+void orc_quantize_absmax_u8(uint8_t* codes, uint16_t* scales, const uint16_t* in, size_t rows,
+                            size_t cols, int block);
+void orc_dequantize_absmax_u8(uint16_t* out, const uint16_t* scales, const uint8_t* codes,
+                              size_t rows, size_t cols, int block);
+
+/* ---- matmul: out[M,N] = lhs[M,K] * rhs[N,K]^T + beta * out ----
+ * flavour 0: llama_cu.cu:111-122 (and 125-145 for u8), one sequential fp32 sum per output.
+ * flavour 1: the tensor-core kernels llama_cu.cu:150-220, 225-285, 294-366: fp16 operands
+ *            (u8 weights first rounded to fp16 by dequantize_absmax_one, 287-289), fp32
+ *            accumulation in an order the hardware fixes; restated with 16 interleaved partial
+ *            sums and a pairwise tree. */
+void orc_matmul_nt(uint16_t* out, const uint16_t* lhs, const uint16_t* rhs, int M, int K, int N,
+                   float beta, int flavour);
+void orc_matmul_nt_u8(uint16_t* out, const uint16_t* lhs, const uint8_t* codes,
+                      const uint16_t* scales, int M, int K, int N, int block, float beta,
+                      int flavour);
+
+/* ---- element-wise and row kernels ---- */
+/* llama_cu.cu:66-107 */
+void orc_rms_norm(uint16_t* out, const uint16_t* in, const uint16_t* weights, int rows, int cols,
+                  float eps);
+/* llama_cu.cu:368-389 */
+void orc_rotary(uint16_t* out, const uint16_t* in, int rows, int cols, int n_heads, int pos_offset,
+                float theta);
+/* llama_cu.cu:400-428; out is [n_heads][n_new][T] with row stride T */
+void orc_matmul_qk(uint16_t* out, const uint16_t* q, const uint16_t* k, int n_new, int T, int dim,
+                   int n_heads, int start_pos);
+/* llama_cu.cu:433-499; rows = product of all leading dimensions */
+void orc_softmax_rows(uint16_t* out, const uint16_t* in, int rows, int w, float temp);
+/* llama_cu.cu:511-531 */
+void orc_matmul_qkv(uint16_t* out, const uint16_t* p, const uint16_t* v, int n_new, int T, int dim,
+                    int n_heads);
+/* llama_cu.cu:533-539 */
+void orc_silu_mul(uint16_t* out, const uint16_t* a, const uint16_t* b, size_t size);
+/* llama_cu.cu:32-44 and 46-62 */
+void orc_embed(uint16_t* out, const int16_t* ids, int n_ids, int dim, const uint16_t* table);
+void orc_embed_u8(uint16_t* out, const int16_t* ids, int n_ids, int dim, const uint8_t* table,
+                  const uint16_t* scales, int block);
+/* llama_cu.cu:1205-1209: first maximum of fp16 values compared as float */
+int orc_argmax_first(const uint16_t* probs, int n);
+
+/* ---- whole model: llama_cu.cu:882-1210 with seeded random weights instead of files ---- */
+typedef struct orc_model orc_model;
+typedef struct orc_context orc_context;
+
+/* q_type 0 = fp16, 1 = uint8 (weights generated in fp16, then quantised with block `qblock`).
+ * Weight streams: tok_embeddings 1, output 2, layer l: 16+16*l + {wq 0, wk 1, wv 2, wo 3, w1 4,
+ * w2 5, w3 6}; every matrix ~N(0, weight_std); all norm weights are 1.0. */
+orc_model* orc_model_create(int dim, int multiple_of, int n_heads, int n_layers, int n_vocab,
+                            float norm_eps, int q_type, int qblock, uint64_t seed,
+                            float weight_std);
+void orc_model_destroy(orc_model*);
+int orc_model_ffn_dim(const orc_model*);
+/* borrowed pointers into the model for cross-checks: which = stream id as above, scales may be
+ * NULL for fp16 models */
+const void* orc_model_tensor(const orc_model*, uint64_t stream, const uint16_t** scales);
+
+/* literal_rope 1 = keep K unrotated and re-rotate all cached rows on every call, exactly as
+ * llama_cu.cu:1150-1153; 0 = rotate once when the row is written (same bits, cheaper). */
+orc_context* orc_context_create(orc_model*, int context_len, float temperature, int matmul_flavour,
+                                int literal_rope);
+void orc_context_destroy(orc_context*);
+void orc_context_clear(orc_context*);
+int orc_context_start_pos(const orc_context*);
+/* llama_cu.cu:1073-1210.  Optional outputs (may be NULL): hidden = residual stream after the last
+ * layer [n][dim]; logits = fp16 logits of the last row [n_vocab]; probs = softmax(temp) [n_vocab]. */
+int orc_context_next_token(orc_context*, const int16_t* tokens, int n, uint16_t* hidden,
+                           uint16_t* logits, uint16_t* probs);
+/* borrowed KV rows of one layer, [context_len][dim]; K is returned rotated */
+void orc_context_kv(orc_context*, int layer, uint16_t* k_rot, uint16_t* v, int T);
+
+int orc_num_threads(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,245 @@
+"""Pins the oracle's restatement of the reference kernels (llama_cu.cu:30-540) by what the
+mathematics fixes: float64 brute force written independently in numpy, exact special cases,
+and invariants.  Each check is chosen so that a dropped term, a wrong index or a transposed
+operand fails it."""
+import numpy as np
+import pytest
+
+import oracle_lib as O
+
+RNG = np.random.default_rng(1234)
+
+
+def rel_err(a, ref):
+    a = np.asarray(a, dtype=np.float64)
+    ref = np.asarray(ref, dtype=np.float64)
+    return np.max(np.abs(a - ref)) / max(np.max(np.abs(ref)), 1e-30)
+
+
+def f16(a):
+    return np.asarray(a, dtype=np.float32).astype(np.float16)
+
+
+# ------------------------------------------------------------------ matmul
+@pytest.mark.parametrize("flavour", [0, 1])
+@pytest.mark.parametrize("M,K,N", [(1, 256, 64), (5, 272, 33), (16, 1024, 128), (3, 40, 7)])
+def test_matmul_vs_float64(flavour, M, K, N):
+    x = f16(RNG.normal(0, 1, (M, K)))
+    w = f16(RNG.normal(0, 0.02, (N, K)))
+    out = O.matmul_nt(x, w, flavour=flavour)
+    ref = x.astype(np.float64) @ w.astype(np.float64).T
+    # fp32 accumulation + one fp16 rounding
+    assert np.max(np.abs(out.astype(np.float64) - ref)) <= np.max(np.abs(ref)) * 2.0 ** -10
+
+
+@pytest.mark.parametrize("flavour", [0, 1])
+def test_matmul_exact_cases(flavour):
+    K = 128
+    x = f16(RNG.normal(0, 1, (4, K)))
+    eye = np.eye(K, dtype=np.float16)
+    assert (O.matmul_nt(x, eye, flavour=flavour).view(np.uint16) == x.view(np.uint16)).all()
+    w = f16(RNG.normal(0, 0.02, (48, K)))
+    onehot = np.zeros((1, K), dtype=np.float16)
+    onehot[0, 37] = 1
+    assert (O.matmul_nt(onehot, w, flavour=flavour)[0].view(np.uint16) == w[:, 37].view(np.uint16)).all()
+    # asymmetric operand: out[m, n] pairs lhs row m with rhs row n (a transposed operand fails)
+    w2 = np.zeros((3, K), dtype=np.float16)
+    w2[2, 5] = 2
+    x2 = np.zeros((2, K), dtype=np.float16)
+    x2[1, 5] = 3
+    out = O.matmul_nt(x2, w2, flavour=flavour)
+    assert out[1, 2] == 6 and np.count_nonzero(out) == 1
+
+
+@pytest.mark.parametrize("flavour", [0, 1])
+def test_matmul_beta_residual(flavour):
+    x = f16(RNG.normal(0, 1, (3, 256)))
+    w = f16(RNG.normal(0, 0.02, (20, 256)))
+    old = f16(RNG.normal(0, 1, (3, 20)))
+    out = O.matmul_nt(x, w, beta=1.0, out=old, flavour=flavour)
+    ref = x.astype(np.float64) @ w.astype(np.float64).T + old.astype(np.float64)
+    assert np.max(np.abs(out.astype(np.float64) - ref)) <= np.max(np.abs(ref)) * 2.0 ** -10
+    # beta = 0 ignores whatever the output held
+    junk = np.full((3, 20), np.inf, dtype=np.float16)
+    assert np.isfinite(O.matmul_nt(x, w, beta=0.0, out=junk, flavour=flavour)).all()
+
+
+@pytest.mark.parametrize("flavour", [0, 1])
+def test_matmul_u8_vs_float64_and_dequant_route(flavour):
+    K, N, M, block = 512, 40, 3, 128
+    w = f16(RNG.normal(0, 0.02, (N, K)))
+    x = f16(RNG.normal(0, 1, (M, K)))
+    codes, scales = O.quantize_absmax_u8(w, block)
+    out = O.matmul_nt_u8(x, codes, scales, block, flavour=flavour)
+    wd64 = (codes.astype(np.float64) - 127.5) * np.repeat(scales.astype(np.float64), block, axis=1)
+    ref = x.astype(np.float64) @ wd64.T
+    assert np.max(np.abs(out.astype(np.float64) - ref)) <= np.max(np.abs(ref)) * 2.0 ** -9
+    if flavour == 1:
+        # the tensor-core route is exactly "dequantise to fp16, then the fp16 matmul" (llama_cu.cu:331-342)
+        wd = O.dequantize_absmax_u8(codes, scales, block)
+        assert (O.matmul_nt(x, wd, flavour=1).view(np.uint16) == out.view(np.uint16)).all()
+
+
+def test_matmul_row_independence():
+    x = f16(RNG.normal(0, 1, (9, 256)))
+    w = f16(RNG.normal(0, 0.02, (31, 256)))
+    full = O.matmul_nt(x, w)
+    for r in (0, 4, 8):
+        assert (O.matmul_nt(x[r:r + 1], w).view(np.uint16) == full[r:r + 1].view(np.uint16)).all()
+
+
+# ------------------------------------------------------------------ rms norm
+def test_rms_norm_closed_forms():
+    cols = 512
+    ones = np.ones(cols, dtype=np.float16)
+    const = np.full((2, cols), 3.0, dtype=np.float16)
+    const[1] = -0.25
+    out = O.rms_norm(const, ones, 0.0)
+    assert (out[0] == 1.0).all() and (out[1] == -1.0).all()
+    x = f16(RNG.normal(0, 1, (7, cols)))
+    w = f16(RNG.normal(1, 0.1, cols))
+    out = O.rms_norm(x, w, 1e-6)
+    x64 = x.astype(np.float64)
+    inner = (x64 / np.sqrt((x64 ** 2).mean(axis=1, keepdims=True) + 1e-6))
+    ref = w.astype(np.float64) * inner
+    assert rel_err(out, ref) < 2e-3  # two fp16 roundings
+    # the two roundings happen in this order: fp16(x * rms_inv), then fp16(w * that)
+    inner16 = inner.astype(np.float32).astype(np.float16)
+    two_step = (w.astype(np.float32) * inner16.astype(np.float32)).astype(np.float16)
+    assert (two_step.view(np.uint16) != out.view(np.uint16)).mean() < 0.01
+    # scale invariance (eps = 0): norm(4x) == norm(x) exactly, powers of two commute with rounding
+    assert (O.rms_norm(x * np.float16(4), w, 0.0).view(np.uint16) == O.rms_norm(x, w, 0.0).view(np.uint16)).all()
+
+
+# ------------------------------------------------------------------ rotary
+def test_rotary_properties():
+    n_heads, head_dim = 4, 128
+    dim = n_heads * head_dim
+    x = f16(RNG.normal(0, 1, (6, dim)))
+    r0 = O.rotary(x[:1], n_heads, pos_offset=0)
+    assert (r0.view(np.uint16) == x[:1].view(np.uint16)).all()  # position 0 is the identity
+    pos0 = 11
+    out = O.rotary(x, n_heads, pos_offset=pos0).astype(np.float64)
+    z = x.astype(np.float64).reshape(6, n_heads, head_dim // 2, 2)
+    zc = z[..., 0] + 1j * z[..., 1]
+    pos = (pos0 + np.arange(6))[:, None, None]
+    freq = 1.0 / (10000.0 ** (np.arange(0, head_dim, 2) / head_dim))[None, None, :]
+    ref = zc * np.exp(1j * pos * freq)
+    got = out.reshape(6, n_heads, head_dim // 2, 2)
+    gc = got[..., 0] + 1j * got[..., 1]
+    assert np.max(np.abs(gc - ref)) < 4e-3  # fp32 angle at pos<=16 plus fp16 rounding
+    assert np.max(np.abs(np.abs(gc) - np.abs(zc))) < 4e-3  # pair norm preserved
+    # pair 0 of every head turns by exactly `pos` radians
+    ang = np.angle(gc[:, :, 0] / zc[:, :, 0])
+    want = np.angle(np.exp(1j * (pos0 + np.arange(6))))[:, None]
+    assert np.max(np.abs(np.angle(np.exp(1j * (ang - want))))) < 5e-3
+
+
+# ------------------------------------------------------------------ softmax
+def test_softmax_properties():
+    for w in (7, 256, 1000):
+        u = np.full((3, w), 1.5, dtype=np.float16)
+        out = O.softmax_rows(u)
+        assert (out.view(np.uint16) == np.float16(np.float32(1.0) / np.float32(w)).view(np.uint16)).all()
+    x = f16(RNG.normal(0, 2, (5, 777)))
+    x[:, 400:] = -np.inf
+    out = O.softmax_rows(x)
+    assert (out[:, 400:] == 0).all()
+    x64 = x[:, :400].astype(np.float64)
+    e = np.exp(x64 - x64.max(axis=1, keepdims=True))
+    ref = e / e.sum(axis=1, keepdims=True)
+    assert np.max(np.abs(out[:, :400].astype(np.float64) - ref)) <= ref.max() * 2.0 ** -10
+    assert np.all(np.abs(out.astype(np.float64).sum(axis=1) - 1) < 2e-3)
+    # temperature divides the logits
+    t = O.softmax_rows(x, temp=0.8)
+    e = np.exp(x64 / np.float64(np.float32(0.8)) - (x64 / np.float64(np.float32(0.8))).max(axis=1, keepdims=True))
+    ref = e / e.sum(axis=1, keepdims=True)
+    assert np.max(np.abs(t[:, :400].astype(np.float64) - ref)) <= ref.max() * 2.0 ** -10
+    # 3-d input: every leading index is a row
+    y = f16(RNG.normal(0, 1, (2, 3, 50)))
+    assert (O.softmax_rows(y).reshape(6, 50).view(np.uint16) == O.softmax_rows(y.reshape(6, 50)).view(np.uint16)).all()
+
+
+# ------------------------------------------------------------------ attention
+def np_attention64(q, k, v, n_heads, start_pos):
+    n, dim = q.shape
+    T = k.shape[0]
+    hd = dim // n_heads
+    out = np.zeros((n, dim))
+    for h in range(n_heads):
+        qs, ks, vs = (a[:, h * hd:(h + 1) * hd].astype(np.float64) for a in (q, k, v))
+        s = qs @ ks.T / np.sqrt(hd)
+        mask = np.arange(T)[None, :] > (np.arange(n)[:, None] + start_pos)
+        s[mask] = -np.inf
+        p = np.exp(s - s.max(axis=1, keepdims=True))
+        p /= p.sum(axis=1, keepdims=True)
+        out[:, h * hd:(h + 1) * hd] = p @ vs
+    return out
+
+
+@pytest.mark.parametrize("n,T,start", [(5, 5, 0), (1, 9, 8), (3, 10, 7)])
+def test_attention_vs_float64(n, T, start):
+    n_heads, hd = 3, 32
+    dim = n_heads * hd
+    q = f16(RNG.normal(0, 1, (n, dim)))
+    k = f16(RNG.normal(0, 1, (T, dim)))
+    v = f16(RNG.normal(0, 1, (T, dim)))
+    out = O.attention(q, k, v, n_heads, start)
+    ref = np_attention64(q, k, v, n_heads, start)
+    assert np.max(np.abs(out.astype(np.float64) - ref)) < 4e-3
+    s = O.matmul_qk(q, k, n_heads, start)
+    assert s.shape == (n_heads, n, T)
+    for r in range(n):
+        assert np.isneginf(s[:, r, r + start + 1:]).all() and np.isfinite(s[:, r, :r + start + 1]).all()
+    # the 1/sqrt(head_dim) scale and the head slicing
+    h = 2
+    want = q[0, h * hd:(h + 1) * hd].astype(np.float64) @ k[0, h * hd:(h + 1) * hd].astype(np.float64) / np.sqrt(hd)
+    assert abs(float(s[h, 0, 0]) - want) <= abs(want) * 2.0 ** -10 + 1e-6
+
+
+def test_attention_first_row_is_v0():
+    n_heads, hd, n = 2, 64, 4
+    dim = n_heads * hd
+    q, k, v = (f16(RNG.normal(0, 1, (n, dim))) for _ in range(3))
+    out = O.attention(q, k, v, n_heads, 0)
+    assert (out[0].view(np.uint16) == v[0].view(np.uint16)).all()  # causal row 0 sees only itself, p = 1
+
+
+def test_decode_equals_last_prefill_row():
+    n_heads, hd, T = 2, 64, 12
+    dim = n_heads * hd
+    q, k, v = (f16(RNG.normal(0, 1, (T, dim))) for _ in range(3))
+    full = O.attention(q, k, v, n_heads, 0)
+    last = O.attention(q[-1:], k, v, n_heads, T - 1)
+    assert (full[-1:].view(np.uint16) == last.view(np.uint16)).all()
+
+
+# ------------------------------------------------------------------ silu, embed, argmax
+def test_silu_mul():
+    a = f16(RNG.normal(0, 2, 5000))
+    b = f16(RNG.normal(0, 1, 5000))
+    out = O.silu_mul(a, b)
+    a64, b64 = a.astype(np.float64), b.astype(np.float64)
+    ref = a64 / (1 + np.exp(-a64)) * b64
+    assert np.max(np.abs(out.astype(np.float64) - ref)) <= np.max(np.abs(ref)) * 2.0 ** -10
+    z = O.silu_mul(np.zeros(4, dtype=np.float16), b[:4])
+    assert (z == 0).all()
+    big = O.silu_mul(np.array([20.0, -20.0], dtype=np.float16), np.array([1.0, 1.0], dtype=np.float16))
+    assert big[0] == 20.0 and abs(float(big[1])) < 1e-6
+
+
+def test_embed_and_embed_u8():
+    table = f16(RNG.normal(0, 0.02, (50, 256)))
+    ids = [3, 49, 0, 3]
+    out = O.embed(ids, table)
+    assert (out.view(np.uint16) == table[ids].view(np.uint16)).all()
+    codes, scales = O.quantize_absmax_u8(table, 128)
+    out8 = O.embed_u8(ids, codes, scales, 128)
+    assert (out8.view(np.uint16) == O.dequantize_absmax_u8(codes, scales, 128)[ids].view(np.uint16)).all()
+
+
+def test_argmax_first_wins():
+    p = np.array([0.1, 0.5, 0.2, 0.5, 0.5], dtype=np.float16)
+    assert O.argmax_first(p) == 1
+    assert O.argmax_first(np.array([0.0, -0.0], dtype=np.float16)) == 0
+    assert O.argmax_first(np.array([1, 2, 3], dtype=np.float16)) == 2

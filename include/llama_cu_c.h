@@ -1,0 +1,56 @@
+/*
+ * C handles over the C++ host interface (llama_cu_host.hpp), for callers that cannot include
+ * C++ headers: the Python tests and bench.py bind these with ctypes.  Each function names the
+ * llama_cu.h member of the reference it forwards to.  Return conventions: pointers are NULL on
+ * failure; int functions return 0 / a value >= 0 on success and a negative number on failure.
+ * A failing GPU call inside the host layer prints the error and raises SIGSEGV, as the
+ * reference's CHECK_CUDA does (llama_cu.h:48-56).
+ */
+#ifndef LLAMA_CU_C_H
+#define LLAMA_CU_C_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct lcu_model lcu_model;
+typedef struct lcu_context lcu_context;
+
+/* llama_params (llama_cu.h:280-291) from its fields; q_type 0 = fp16, 1 = uint8 */
+/* llama_model::create_synthetic (no reference counterpart: seeded random weights, norms = 1) */
+lcu_model* lcu_model_create_synthetic(uint32_t dim, uint32_t multiple_of, uint32_t n_heads, uint32_t n_layers,
+                                      uint32_t n_vocab, float norm_eps, int q_type, int quantization_block_size,
+                                      uint64_t seed, float weight_std);
+/* mapped_buffer(path + "/params") + llama_params::load + llama_partition::autopipe + llama_model::load
+ * (main.cpp:24-57, llama_cu.cu:987-997) */
+lcu_model* lcu_model_load(const char* model_dir, int context_len);
+void lcu_model_destroy(lcu_model*);
+uint32_t lcu_model_ffn_dim(const lcu_model*);                      /* llama_params::ffn_dim */
+/* copies a weight matrix back to the host: stream id 1 tok_embeddings, 2 output, 16+16l+{0..6}
+ * wq wk wv wo w1 w2 w3; `scales` may be NULL for fp16 models */
+int lcu_model_read_tensor(const lcu_model*, uint64_t stream_id, void* values, void* scales);
+
+lcu_context* lcu_context_create(lcu_model*, int context_len, float temperature);   /* llama_context::create */
+void lcu_context_destroy(lcu_context*);
+void lcu_context_clear_tokens(lcu_context*);                                        /* clear_tokens */
+size_t lcu_context_memory_usage(lcu_context*);                                      /* context_memory_usage */
+size_t lcu_context_tokens_left(lcu_context*);                                       /* tokens_left */
+/* next_token (llama_cu.h:380); -1 if the tokens do not fit the context or an id is out of range */
+int lcu_context_next_token(lcu_context*, const int16_t* tokens, int n);
+/* results of the last next_token call, fp16: logits and probabilities [n_vocab], the residual
+ * stream after the last layer [n][dim] (rows = n of that call) */
+int lcu_context_read_logits(lcu_context*, uint16_t* out);
+int lcu_context_read_probs(lcu_context*, uint16_t* out);
+int lcu_context_read_hidden(lcu_context*, uint16_t* out, int rows);
+/* first T rows of one layer's KV cache, [T][dim] each; K is stored rotated */
+int lcu_context_read_kv(lcu_context*, int layer, uint16_t* k_out, uint16_t* v_out, int T);
+/* the hipStream_t (as void*) the context launches on, for event timing */
+void* lcu_context_stream(lcu_context*);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,147 @@
+/*
+ * C ABI of the MI355X (gfx950) device layer behind the llama_cu host interface.
+ *
+ * The reference (eiz/llama.cu) has no FFI: its forward pass, llama_context_impl::next_token
+ * (llama_cu.cu:1073-1210), launches CUDA kernels directly.  This header declares one entry point
+ * per launch site of that function, plus the buffer calls of llama_cu.h:109-134, so that the host
+ * code (and any other language) reaches the GPU through plain pointers and sizes.
+ *
+ * Conventions
+ *   - every pointer named *_dev is device memory; fp16 tensors are IEEE binary16, row-major
+ *   - `stream` is a hipStream_t passed as void* (NULL = the default stream); work is asynchronous
+ *     unless stated
+ *   - every function returns 0 on success and a negative code on failure, never throws, never
+ *     exits; lcu_last_error() describes the last failure of the calling thread
+ *   - shapes the kernels do not support are rejected before any launch (LCU_E_SHAPE)
+ *   - one host thread per stream; the library keeps no global mutable state besides per-device
+ *     workspaces created by lcu_init
+ */
+#ifndef LLAMA_CU_HIP_H
+#define LLAMA_CU_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define LCU_OK 0
+#define LCU_E_HIP (-1)      /* a HIP runtime call failed */
+#define LCU_E_SHAPE (-2)    /* unsupported or inconsistent shape / null pointer */
+#define LCU_E_NOINIT (-3)   /* lcu_init has not run on this device */
+
+typedef struct lcu_device_props {
+  char name[128];
+  int compute_units;
+  int lds_bytes_per_block;
+  int l2_bytes;
+  int clock_khz;
+  int memory_clock_khz;
+  int memory_bus_bits;
+  size_t total_memory;
+  size_t free_memory;
+} lcu_device_props;
+
+/* ---- runtime: llama_cu.cu:1525-1542 (initialize), 691-736 (scoped_gpu, gpu_buffer[_view]) ---- */
+int lcu_init(int device);
+const char* lcu_last_error(void);
+int lcu_device_get_props(int device, lcu_device_props* out);
+int lcu_get_device(int* out_device);                                            /* scoped_gpu, 691-697 */
+int lcu_set_device(int device);
+int lcu_malloc(void** out_dev, size_t bytes);                                   /* gpu_buffer ctor, 712-715 */
+int lcu_free(void* dev);                                                        /* gpu_buffer dtor, 732-736 */
+int lcu_memset(void* dev, int byte_value, size_t bytes, void* stream);          /* llama_cu.h:239-241 */
+int lcu_h2d(void* dst_dev, const void* src_host, size_t bytes, void* stream);   /* copy_from, 699-706; async */
+int lcu_d2h(void* dst_host, const void* src_dev, size_t bytes, void* stream);   /* copy_to, 707-710; blocks */
+int lcu_d2d(void* dst_dev, const void* src_dev, size_t bytes, void* stream);
+int lcu_stream_create(void** out_stream);
+int lcu_stream_destroy(void* stream);
+int lcu_sync(void* stream);                                                     /* NULL = whole device */
+int lcu_event_create(void** out_event);
+int lcu_event_destroy(void* event);
+int lcu_event_record(void* event, void* stream);
+int lcu_event_elapsed_ms(float* out_ms, void* start_event, void* stop_event);   /* waits for stop */
+
+/* ---- matmul: out[M,N] = lhs[M,K] * rhs[N,K]^T + beta * out ----
+ * lcu_gemm_f16_nt replaces matmul_nt(tensor4d_view) and the kernels it selects
+ * (llama_cu.cu:1463-1496, 150-220, 225-285): M == 1 runs the streaming GEMV, larger M the MFMA
+ * GEMM.  K must be a multiple of 8.  fp32 accumulation, one rounding to fp16 of acc + beta*out. */
+int lcu_gemm_f16_nt(void* out_dev, const void* lhs_dev, const void* rhs_dev, int M, int K, int N,
+                    float beta, void* stream);
+/* lcu_gemm_f16u8_nt replaces matmul_nt(generic_tensor&) for quantised weights and
+ * matmul_nt_wmma_16x128x256_fp16u8 (llama_cu.cu:1498-1523, 287-366): codes [N,K] uint8, scales
+ * [N,K/block] fp16, each weight dequantised as fp16((code - 127.5) * scale) before it is used.
+ * K % 16 == 0, block % 16 == 0, K % block == 0. */
+int lcu_gemm_f16u8_nt(void* out_dev, const void* lhs_dev, const void* codes_dev,
+                      const void* scales_dev, int M, int K, int N, int block, float beta,
+                      void* stream);
+
+/* ---- int8 absmax quantiser: transform.cu:28-72 and 74-87; block in {32, 64, 128, 256, 512, 1024} */
+int lcu_quantize_absmax_u8(void* codes_dev, void* scales_dev, const void* in_dev, size_t rows,
+                           size_t cols, int block, void* stream);
+int lcu_dequantize_absmax_u8(void* out_dev, const void* scales_dev, const void* codes_dev,
+                             size_t rows, size_t cols, int block, void* stream);
+
+/* ---- row and element-wise kernels ---- */
+/* rms_norm, llama_cu.cu:66-107 (launch sites 1129, 1176, 1191) */
+int lcu_rmsnorm(void* out_dev, const void* in_dev, const void* weights_dev, int rows, int cols,
+                float eps, void* stream);
+/* rotary, llama_cu.cu:368-389 (launch sites 1146, 1152).  The angles cos/sin(pos / theta^(c/head_dim))
+ * come from a table built once on the host with the C library's powf/cosf/sinf:
+ * table_dev[pos][pair] = {cos, sin} as float2, pair = (c mod head_dim) / 2. */
+int lcu_rope_table_create(void** out_table_dev, int positions, int head_dim, float theta);
+int lcu_rope(void* out_dev, const void* in_dev, int rows, int cols, int n_heads, int pos_offset,
+             const void* table_dev, int table_positions, void* stream);
+/* softmax_rows, llama_cu.cu:433-499 (launch sites 1166, 1196); in place allowed */
+int lcu_softmax_rows(void* out_dev, const void* in_dev, int rows, int w, float temp, void* stream);
+/* silu, llama_cu.cu:533-539 (launch site 1183) */
+int lcu_silu_mul(void* out_dev, const void* a_dev, const void* b_dev, size_t size, void* stream);
+/* embed / embed_uint8, llama_cu.cu:32-62 (launch sites 1090, 1094); ids are int16 */
+int lcu_embed(void* out_dev, const void* ids_dev, int n_ids, int dim, const void* table_dev,
+              int n_vocab, void* stream);
+int lcu_embed_u8(void* out_dev, const void* ids_dev, int n_ids, int dim, const void* codes_dev,
+                 const void* scales_dev, int block, int n_vocab, void* stream);
+/* the host argmax of llama_cu.cu:1205-1209 done on the device: index of the first maximum of n
+ * fp16 values compared as float, written as int32 */
+int lcu_argmax_f16(void* out_index_dev, const void* values_dev, int n, void* stream);
+
+/* ---- attention: matmul_qk + softmax_rows + matmul_qkv, llama_cu.cu:400-531, launch sites
+ * 1161-1171, without the [n_heads, n, T] score tensor in memory.  q [n_new, dim]; k (already
+ * rotated) and v are the first T rows of a [*, dim] cache; causal: row r sees columns
+ * c <= r + start_pos.  Scores are rounded to fp16, probabilities are rounded to fp16, the
+ * weighted sum runs in fp32: the reference's three rounding points.  head_dim must be 128,
+ * T <= 4096. */
+int lcu_attention(void* out_dev, const void* q_dev, const void* k_dev, const void* v_dev,
+                  int n_new, int T, int start_pos, int dim, int n_heads, void* stream);
+
+/* ---- fused decode steps (n_new == 1), each replacing several launch sites of next_token ---- */
+/* rms_norm(x, attn_norm) -> Wq/Wk/Wv GEMV -> RoPE(q, k at position pos) -> q to q_out, k and v into
+ * row pos of the caches: llama_cu.cu:1129-1156.  Weight pointers are fp16 [dim, dim], or uint8 codes
+ * with fp16 scales when block > 0. */
+int lcu_decode_qkv(void* q_out_dev, void* k_cache_dev, void* v_cache_dev, const void* x_dev,
+                   const void* norm_w_dev, const void* wq_dev, const void* wk_dev, const void* wv_dev,
+                   const void* sq_dev, const void* sk_dev, const void* sv_dev, int block, int dim,
+                   int n_heads, int pos, float eps, const void* rope_table_dev, int table_positions,
+                   void* stream);
+/* rms_norm(x, ffn_norm) -> W1 and W3 GEMV -> silu(w1) * w3: llama_cu.cu:1176-1183 */
+int lcu_decode_ffn_up(void* out_dev, const void* x_dev, const void* norm_w_dev, const void* w1_dev,
+                      const void* w3_dev, const void* s1_dev, const void* s3_dev, int block, int dim,
+                      int ffn, float eps, void* stream);
+/* rms_norm(x, norm) -> output GEMV: llama_cu.cu:1191-1195 for the single row that is used */
+int lcu_decode_logits(void* logits_dev, const void* x_dev, const void* norm_w_dev,
+                      const void* wout_dev, const void* sout_dev, int block, int dim, int n_vocab,
+                      float eps, void* stream);
+
+/* ---- synthetic tensors (no counterpart in the reference, which reads weights from files):
+ * value[i] = fp16(float(S - 262140) * scale), S = sum of the eight 16-bit fields of two chained
+ * splitmix64 hashes of (seed, stream_id, i), scale = float(std / sqrt(8 * (65536^2 - 1) / 12)).
+ * Integer-exact, so any host restating the recipe gets the same bits. */
+int lcu_fill_normal_f16(void* out_dev, size_t n, uint64_t seed, uint64_t stream_id, float std,
+                        void* stream);
+int lcu_fill_f16(void* out_dev, size_t n, uint16_t bits, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

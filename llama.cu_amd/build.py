@@ -1,0 +1,48 @@
+"""Builds libllama_cu_amd.so (HIP kernels + C ABI + C++ host layer) for gfx950 with hipcc."""
+import os
+import subprocess
+import sys
+
+PKG = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(PKG)
+LIB = os.path.join(PKG, "libllama_cu_amd.so")
+
+HIP_SOURCES = ["csrc/runtime.hip", "csrc/elementwise.hip", "csrc/gemv.hip", "csrc/gemm.hip", "csrc/attention.hip"]
+HOST_SOURCES = ["host/buffers.cpp", "host/params.cpp", "host/model.cpp", "host/tokenizer.cpp", "host/capi.cpp"]
+
+COMMON = ["-O3", "-std=c++17", "-fPIC", "-I" + os.path.join(ROOT, "include"), "-I" + os.path.join(PKG, "csrc"),
+          "-I" + os.path.join(PKG, "host"), "-Wall", "-Wno-unused-function"]
+# no fast-math, no implicit fma contraction (the kernels write their fused multiply-adds out), and
+# no packed-fp32 instructions
+DEVICE = ["--offload-arch=gfx950", "-ffp-contract=off", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+
+
+def build(verbose=False):
+    objs = []
+    os.makedirs(os.path.join(PKG, "build"), exist_ok=True)
+    procs = []
+    for src in HIP_SOURCES + HOST_SOURCES:
+        obj = os.path.join(PKG, "build", os.path.basename(src) + ".o")
+        objs.append(obj)
+        cmd = ["hipcc"] + COMMON + (DEVICE if src.endswith(".hip") else ["-x", "c++"]) + ["-c", os.path.join(PKG, src), "-o", obj]
+        if verbose:
+            print(" ".join(cmd))
+        procs.append((src, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)))
+    failed = False
+    for src, p in procs:
+        out, _ = p.communicate()
+        out = "\n".join(l for l in out.splitlines() if "packed-fp32-ops" not in l and "unknown target feature" not in l)
+        if p.returncode != 0:
+            failed = True
+            sys.stderr.write("FAILED %s\n%s\n" % (src, out))
+        elif verbose and out.strip():
+            print(out)
+    if failed:
+        raise RuntimeError("hipcc failed")
+    cmd = ["hipcc", "--offload-arch=gfx950", "-shared", "-o", LIB] + objs
+    subprocess.check_call(cmd)
+    return LIB
+
+
+if __name__ == "__main__":
+    print(build(verbose="-v" in sys.argv))

@@ -1,0 +1,321 @@
+// Causal self-attention over the KV cache: the reference's matmul_qk -> softmax_rows -> matmul_qkv
+// chain (llama_cu.cu:400-428, 433-499, 511-531; launch sites 1161-1171) without its
+// [n_heads, n, T] score tensor in memory and without its per-layer cudaMalloc (1120-1122).
+//
+// The reference's three rounding points are kept: scores are rounded to fp16, probabilities are
+// rounded to fp16 after a softmax over the whole row (true row maximum and row sum, no online
+// rescaling), and the probability-weighted sum of V runs in fp32 and is rounded once.
+//
+// Layouts: q [n_new, dim]; k, v = first T rows of a [*, dim] cache (K already rotated); head h is
+// columns h*128 .. h*128+127.
+//
+// Decode (n_new == 1), HBM bound, two kernels so that every compute unit streams part of the cache:
+//   scores: grid (T/256, heads); 16 lanes share one cached K row (16 bytes each), fp32 dot,
+//           fp16 score to a workspace
+//   pv:     grid (T/256, heads); every workgroup redoes the cheap row max / exp-sum over all T
+//           scores of its head, forms its 256 probabilities, accumulates p * V for them, and the
+//           last workgroup of a head to arrive adds the partial sums in split order
+// Prefill (n_new > 1), matrix-core bound: one workgroup per (32 query rows, head); Q.K^T by
+// v_mfma_f32_16x16x32_f16 into an LDS score strip [32][T], softmax in LDS, P.V by MFMA with V
+// staged transposed in LDS.
+#include "common.hpp"
+
+using namespace lcu;
+
+namespace {
+
+constexpr int HD = 128;            // head_dim
+constexpr int MAX_T_DECODE = 4096;
+constexpr int MAX_HEADS = 64;
+constexpr int SPLIT = 256;         // cache rows per decode workgroup
+constexpr int MAX_SPLITS = MAX_T_DECODE / SPLIT;
+
+// workspace carve-up (see lcu_init): scores, partial sums, arrival counters
+constexpr size_t WS_SCORES = 0;
+constexpr size_t WS_PARTIAL = WS_SCORES + (size_t)MAX_HEADS * MAX_T_DECODE * sizeof(half_t);
+constexpr size_t WS_COUNTERS = WS_PARTIAL + (size_t)MAX_HEADS * MAX_SPLITS * HD * sizeof(float);
+constexpr size_t WS_END = WS_COUNTERS + MAX_HEADS * sizeof(int);
+
+__global__ __launch_bounds__(256) void decode_scores_kernel(half_t* __restrict__ scores, const half_t* __restrict__ q,
+                                                            const half_t* __restrict__ k, int T, int dim) {
+  const int h = blockIdx.y;
+  const int tid = threadIdx.x;
+  const int sub = tid & 15, grp = tid >> 4;  // 16 lanes per cache row, 16 rows per pass
+  const half8_t qh = *reinterpret_cast<const half8_t*>(q + h * HD + sub * 8);
+  float qf[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) qf[e] = (float)qh[e];
+  const float denom = sqrtf((float)HD);
+  const int base = blockIdx.x * SPLIT;
+#pragma unroll 4
+  for (int it = 0; it < SPLIT / 16; ++it) {
+    const int p = base + it * 16 + grp;
+    float s = 0.0f;
+    if (p < T) {
+      const half8_t kv = __builtin_nontemporal_load(reinterpret_cast<const half8_t*>(k + (size_t)p * dim + h * HD + sub * 8));
+#pragma unroll
+      for (int e = 0; e < 8; ++e) s = fmaf(qf[e], (float)kv[e], s);
+    }
+#pragma unroll
+    for (int off = 8; off > 0; off >>= 1) s += __shfl_xor(s, off, WAVE);
+    if (sub == 0 && p < T) {
+      scores[(size_t)h * MAX_T_DECODE + p] = round_f16(s / denom);  // llama_cu.cu:425
+    }
+  }
+}
+
+__global__ __launch_bounds__(256) void decode_pv_kernel(half_t* __restrict__ out, const half_t* __restrict__ scores,
+                                                        const half_t* __restrict__ v, float* __restrict__ partial,
+                                                        int* __restrict__ counters, int T, int dim, int nsplit) {
+  __shared__ float red[8];
+  __shared__ float gsum[16][HD];
+  __shared__ int s_last;
+  const int h = blockIdx.y, split = blockIdx.x;
+  const int tid = threadIdx.x;
+  const half_t* srow = scores + (size_t)h * MAX_T_DECODE;
+  // softmax_rows statistics over the whole row (llama_cu.cu:442-493), thread t owning t, t+256, ...
+  float m = -INFINITY;
+  for (int i = tid; i < T; i += 256) m = fmaxf(m, (float)srow[i]);
+  m = block256_max(m, red);
+  float s = 0.0f;
+  for (int i = tid; i < T; i += 256) s += expf((float)srow[i] - m);
+  const float total = block256_sum_ref_order(s, red);
+
+  const int sub = tid & 15, grp = tid >> 4;
+  float acc[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) acc[e] = 0.0f;
+  const int base = split * SPLIT;
+#pragma unroll 4
+  for (int it = 0; it < SPLIT / 16; ++it) {
+    const int p = base + it * 16 + grp;
+    if (p < T) {
+      const float prob = (float)round_f16(expf((float)srow[p] - m) / total);  // rounded as stored, 497
+      const half8_t vv = __builtin_nontemporal_load(reinterpret_cast<const half8_t*>(v + (size_t)p * dim + h * HD + sub * 8));
+#pragma unroll
+      for (int e = 0; e < 8; ++e) acc[e] = fmaf(prob, (float)vv[e], acc[e]);
+    }
+  }
+#pragma unroll
+  for (int e = 0; e < 8; ++e) gsum[grp][sub * 8 + e] = acc[e];
+  __syncthreads();
+  float mine = 0.0f;
+  if (tid < HD) {
+#pragma unroll
+    for (int g = 0; g < 16; ++g) mine += gsum[g][tid];
+  }
+  if (nsplit == 1) {
+    if (tid < HD) out[h * HD + tid] = round_f16(mine);
+    return;
+  }
+  if (tid < HD) partial[((size_t)h * MAX_SPLITS + split) * HD + tid] = mine;
+  __threadfence();  // partial sums visible device-wide before the arrival is counted
+  __syncthreads();
+  if (tid == 0) {
+    const int prev = atomicAdd(&counters[h], 1);
+    s_last = (prev == nsplit - 1);
+    if (s_last) counters[h] = 0;  // ready for the next launch
+  }
+  __syncthreads();
+  if (s_last) {
+    __threadfence();
+    if (tid < HD) {
+      float o = 0.0f;
+      for (int sp = 0; sp < nsplit; ++sp) {
+        o += __builtin_nontemporal_load(&partial[((size_t)h * MAX_SPLITS + sp) * HD + tid]);
+      }
+      out[h * HD + tid] = round_f16(o);  // llama_cu.cu:529
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
+// prefill
+// ---------------------------------------------------------------------------------------------
+constexpr int BR = 32;         // query rows per workgroup
+constexpr int CW = 64;         // cache rows per staged chunk
+constexpr int QLD = HD + 8;    // LDS row stride (halves) of the Q and K tiles
+constexpr int VLD = CW + 8;    // LDS row stride of the transposed V chunk
+constexpr int MAX_T_PREFILL = 2048;
+
+__global__ __launch_bounds__(256) void prefill_attention_kernel(half_t* __restrict__ out, const half_t* __restrict__ q,
+                                                                const half_t* __restrict__ k, const half_t* __restrict__ v,
+                                                                int n_new, int T, int start_pos, int dim, int n_tiles) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  // heavier (later) row tiles first: their causal span is longest
+  const int tile = n_tiles - 1 - blockIdx.x;
+  const int h = blockIdx.y;
+  const int r0 = tile * BR;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  // columns this tile can see: c <= r + start_pos for its last real row
+  const int last_row = min(r0 + BR, n_new) - 1;
+  const int c_end = min(T, last_row + start_pos + 1);
+  const int Tc = (c_end + CW - 1) / CW * CW;
+  const int SLD = Tc + 8;
+
+  half_t* Qs = reinterpret_cast<half_t*>(smem);             // [BR][QLD]
+  half_t* KVs = Qs + BR * QLD;                              // K chunk [CW][QLD] or V^T chunk [HD][VLD]
+  half_t* Ss = KVs + (CW * QLD > HD * VLD ? CW * QLD : HD * VLD);  // [BR][SLD]
+
+  // Q tile
+  for (int c = tid; c < BR * HD / 8; c += 256) {
+    const int row = c >> 4, col = (c & 15) * 8;
+    const int gr = r0 + row;
+    half8_t val = (half8_t)(0.0f);
+    if (gr < n_new) val = *reinterpret_cast<const half8_t*>(q + (size_t)gr * dim + h * HD + col);
+    *reinterpret_cast<half8_t*>(&Qs[row * QLD + col]) = val;
+  }
+
+  const float denom = sqrtf((float)HD);
+  const int frow = lane & 15, fk = (lane >> 4) * 8;
+  // ---- scores: S[BR][Tc] = Q . K^T, wave w owns the 16 columns w*16.. of every 64-column chunk
+  for (int c0 = 0; c0 < Tc; c0 += CW) {
+    __syncthreads();
+    for (int c = tid; c < CW * HD / 8; c += 256) {
+      const int row = c >> 4, col = (c & 15) * 8;
+      const int gp = c0 + row;
+      half8_t val = (half8_t)(0.0f);
+      if (gp < T) val = *reinterpret_cast<const half8_t*>(k + (size_t)gp * dim + h * HD + col);
+      *reinterpret_cast<half8_t*>(&KVs[row * QLD + col]) = val;
+    }
+    __syncthreads();
+    float4_t acc[2] = {(float4_t)(0.0f), (float4_t)(0.0f)};
+#pragma unroll
+    for (int ks = 0; ks < HD; ks += 32) {
+      const half8_t fb = *reinterpret_cast<const half8_t*>(&KVs[(wave * 16 + frow) * QLD + ks + fk]);
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        const half8_t fa = *reinterpret_cast<const half8_t*>(&Qs[(i * 16 + frow) * QLD + ks + fk]);
+        acc[i] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fa, fb, acc[i], 0, 0, 0);
+      }
+    }
+    // accumulator register e of lane l is (row 4*(l/16) + e, column l%16)
+    const int col = c0 + wave * 16 + (lane & 15);
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const int row = i * 16 + (lane >> 4) * 4 + e;
+        const bool masked = col > r0 + row + start_pos;  // llama_cu.cu:415
+        Ss[row * SLD + col] = masked ? (half_t)(-INFINITY) : round_f16(acc[i][e] / denom);
+      }
+    }
+  }
+  __syncthreads();
+
+  // ---- softmax over each row of the strip (llama_cu.cu:433-499): wave w owns rows w*8 .. w*8+7
+  for (int rr = 0; rr < BR / 4; ++rr) {
+    half_t* srow = Ss + (wave * (BR / 4) + rr) * SLD;
+    float m = -INFINITY;
+    for (int i = lane; i < Tc; i += WAVE) m = fmaxf(m, (float)srow[i]);
+    m = wave_max(m);
+    float s = 0.0f;
+    for (int i = lane; i < Tc; i += WAVE) s += expf((float)srow[i] - m);
+    s = wave_sum(s);
+    for (int i = lane; i < Tc; i += WAVE) srow[i] = round_f16(expf((float)srow[i] - m) / s);
+  }
+
+  // ---- out[BR][HD] = P . V: wave w owns output columns w*32 .. w*32+31 (two 16-wide tiles)
+  float4_t o[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+#pragma unroll
+    for (int j = 0; j < 2; ++j) o[i][j] = (float4_t)(0.0f);
+  }
+  for (int c0 = 0; c0 < Tc; c0 += CW) {
+    __syncthreads();
+    // V chunk, transposed on the way into LDS: KVs[d][pos]
+    for (int c = tid; c < CW * HD / 8; c += 256) {
+      const int row = c >> 4, col = (c & 15) * 8;
+      const int gp = c0 + row;
+      half8_t val = (half8_t)(0.0f);
+      if (gp < T) val = *reinterpret_cast<const half8_t*>(v + (size_t)gp * dim + h * HD + col);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) KVs[(col + e) * VLD + row] = val[e];
+    }
+    __syncthreads();
+#pragma unroll
+    for (int ks = 0; ks < CW; ks += 32) {
+      half8_t fa[2], fb[2];
+#pragma unroll
+      for (int i = 0; i < 2; ++i) fa[i] = *reinterpret_cast<const half8_t*>(&Ss[(i * 16 + frow) * SLD + c0 + ks + fk]);
+#pragma unroll
+      for (int j = 0; j < 2; ++j) fb[j] = *reinterpret_cast<const half8_t*>(&KVs[(wave * 32 + j * 16 + frow) * VLD + ks + fk]);
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+#pragma unroll
+        for (int j = 0; j < 2; ++j) o[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fa[i], fb[j], o[i][j], 0, 0, 0);
+      }
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int col = h * HD + wave * 32 + j * 16 + (lane & 15);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const int gr = r0 + i * 16 + (lane >> 4) * 4 + e;
+        if (gr < n_new) out[(size_t)gr * dim + col] = round_f16(o[i][j][e]);  // llama_cu.cu:529
+      }
+    }
+  }
+}
+
+size_t prefill_lds_bytes(int Tc) {
+  const size_t kv = (size_t)(CW * QLD > HD * VLD ? CW * QLD : HD * VLD);
+  return ((size_t)BR * QLD + kv + (size_t)BR * (Tc + 8)) * sizeof(half_t);
+}
+
+}  // namespace
+
+extern "C" {
+
+int lcu_attention(void* out_dev, const void* q_dev, const void* k_dev, const void* v_dev, int n_new, int T,
+                  int start_pos, int dim, int n_heads, void* stream) {
+  LCU_REQUIRE(out_dev && q_dev && k_dev && v_dev, "lcu_attention: null pointer");
+  LCU_REQUIRE(n_new >= 0 && start_pos >= 0 && T == start_pos + n_new,
+              "lcu_attention: T (%d) must equal start_pos (%d) + n_new (%d)", T, start_pos, n_new);
+  LCU_REQUIRE(n_heads > 0 && n_heads <= MAX_HEADS && dim == n_heads * HD,
+              "lcu_attention: dim %d / heads %d unsupported (head_dim must be 128, at most %d heads)", dim, n_heads,
+              MAX_HEADS);
+  if (n_new == 0) return LCU_OK;
+  device_state* st = current_device_state();
+  if (!st || !st->ready) return set_error(LCU_E_NOINIT, "lcu_attention: lcu_init has not run on this device");
+  hipStream_t s = as_stream(stream);
+  if (n_new == 1) {
+    LCU_REQUIRE(T <= MAX_T_DECODE, "lcu_attention: T %d exceeds %d", T, MAX_T_DECODE);
+    static_assert(WS_END <= (4u << 20), "workspace too small");
+    unsigned char* ws = (unsigned char*)st->workspace;
+    half_t* scores = (half_t*)(ws + WS_SCORES);
+    float* partial = (float*)(ws + WS_PARTIAL);
+    int* counters = (int*)(ws + WS_COUNTERS);
+    const int nsplit = (T + SPLIT - 1) / SPLIT;
+    dim3 grid(nsplit, n_heads);
+    decode_scores_kernel<<<grid, 256, 0, s>>>(scores, (const half_t*)q_dev, (const half_t*)k_dev, T, dim);
+    LCU_LAUNCH_CHECK();
+    decode_pv_kernel<<<grid, 256, 0, s>>>((half_t*)out_dev, scores, (const half_t*)v_dev, partial, counters, T, dim,
+                                          nsplit);
+    LCU_LAUNCH_CHECK();
+    return LCU_OK;
+  }
+  LCU_REQUIRE(T <= MAX_T_PREFILL, "lcu_attention: T %d exceeds %d for n_new > 1", T, MAX_T_PREFILL);
+  const int n_tiles = (n_new + BR - 1) / BR;
+  const int Tc_max = (T + CW - 1) / CW * CW;
+  const size_t lds = prefill_lds_bytes(Tc_max);
+  static bool attr_set[16] = {};
+  int dev = 0;
+  LCU_HIP(hipGetDevice(&dev));
+  if (!attr_set[dev & 15]) {
+    LCU_HIP(hipFuncSetAttribute((const void*)prefill_attention_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                (int)prefill_lds_bytes(MAX_T_PREFILL)));
+    attr_set[dev & 15] = true;
+  }
+  dim3 grid(n_tiles, n_heads);
+  prefill_attention_kernel<<<grid, 256, lds, s>>>((half_t*)out_dev, (const half_t*)q_dev, (const half_t*)k_dev,
+                                                  (const half_t*)v_dev, n_new, T, start_pos, dim, n_tiles);
+  LCU_LAUNCH_CHECK();
+  return LCU_OK;
+}
+
+}  // extern "C"

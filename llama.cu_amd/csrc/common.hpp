@@ -1,0 +1,116 @@
+// Shared device helpers and the error plumbing of the C ABI.  gfx950 only: 64-wide wavefronts.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+
+#include "llama_cu_hip.h"
+
+namespace lcu {
+
+typedef _Float16 half_t;
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+typedef float float4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t uint4_t __attribute__((ext_vector_type(4)));
+typedef float float16_t __attribute__((ext_vector_type(16)));
+
+constexpr int WAVE = 64;
+
+int set_error(int code, const char* fmt, ...) __attribute__((format(printf, 2, 3)));
+inline hipStream_t as_stream(void* s) { return reinterpret_cast<hipStream_t>(s); }
+
+#define LCU_HIP(expr)                                                                         \
+  do {                                                                                        \
+    hipError_t e__ = (expr);                                                                  \
+    if (e__ != hipSuccess) {                                                                  \
+      return lcu::set_error(LCU_E_HIP, "%s:%d: %s failed: %s", __FILE__, __LINE__, #expr,     \
+                            hipGetErrorString(e__));                                          \
+    }                                                                                         \
+  } while (0)
+
+#define LCU_REQUIRE(cond, ...)                          \
+  do {                                                  \
+    if (!(cond)) {                                      \
+      return lcu::set_error(LCU_E_SHAPE, __VA_ARGS__);  \
+    }                                                   \
+  } while (0)
+
+#define LCU_LAUNCH_CHECK() LCU_HIP(hipGetLastError())
+
+// per-device workspace created by lcu_init (attention partial results and counters)
+struct device_state {
+  bool ready = false;
+  int compute_units = 0;
+  void* workspace = nullptr;
+  size_t workspace_bytes = 0;
+};
+device_state* current_device_state();
+
+// fp32 -> fp16, round to nearest even, as a separate step.  Written through an opaque register so
+// the compiler cannot merge the conversion into the preceding multiply or fused multiply-add
+// (v_fma_mixlo_f16 rounds the exact result once to fp16; the reference rounds to fp32 first, and a
+// value that lands on an fp16 tie after the fp32 rounding then differs by one ulp).
+__device__ __forceinline__ half_t round_f16(float f) {
+  asm("" : "+v"(f));
+  return (half_t)f;
+}
+
+// ---- wavefront reductions (all 64 lanes end with the result) ----
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) {
+    v += __shfl_xor(v, off, WAVE);
+  }
+  return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) {
+    v = fmaxf(v, __shfl_xor(v, off, WAVE));
+  }
+  return v;
+}
+
+// Sum over a 256-thread block of one partial per thread, associated exactly as the reference's
+// block reduction (llama_cu.cu:81-100 and 476-493): groups of 32 consecutive threads reduce by
+// xor distances 16..1, then the eight group sums reduce by xor distances 4, 2, 1.  `red` is 8
+// floats of LDS.  Every thread returns the total.
+__device__ __forceinline__ float block256_sum_ref_order(float v, float* red) {
+#pragma unroll
+  for (int off = 16; off > 0; off >>= 1) {
+    v += __shfl_xor(v, off, WAVE);
+  }
+  const int tid = threadIdx.x;
+  __syncthreads();  // protects `red` against a previous use
+  if ((tid & 31) == 0) {
+    red[tid >> 5] = v;
+  }
+  __syncthreads();
+  float w = red[tid & 7];
+#pragma unroll
+  for (int off = 4; off > 0; off >>= 1) {
+    w += __shfl_xor(w, off, WAVE);
+  }
+  return w;
+}
+
+__device__ __forceinline__ float block256_max(float v, float* red) {
+  v = wave_max(v);
+  const int tid = threadIdx.x;
+  __syncthreads();
+  if ((tid & 63) == 0) {
+    red[tid >> 6] = v;
+  }
+  __syncthreads();
+  return fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+}
+
+// fp16((code - 127.5) * scale): the product is exact in fp32 (9 x 11 significant bits), so this
+// is one rounding, as dequantize_absmax_one (llama_cu.cu:287-289).
+__device__ __forceinline__ half_t dequant_one(uint32_t code, float scale) {
+  return round_f16(((float)code - 127.5f) * scale);
+}
+
+}  // namespace lcu

@@ -1,0 +1,415 @@
+// Row-wise and element-wise kernels of the forward pass, the int8 absmax quantiser, and the
+// synthetic-tensor fill.  Each kernel keeps the reference's fp16 rounding points; reference
+// lines are cited per kernel.
+#include "common.hpp"
+
+using namespace lcu;
+
+namespace {
+
+// ---------------------------------------------------------------------------------------------
+// rms_norm, llama_cu.cu:66-107.  One 256-thread block per row; the sum of squares is associated
+// exactly as the reference's (thread t owns elements t, t+256, ...; see block256_sum_ref_order).
+// Two roundings: fp16(x * rms_inv), then fp16(weight * that).
+// ---------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void rmsnorm_kernel(half_t* __restrict__ out, const half_t* __restrict__ in,
+                                                      const half_t* __restrict__ weights, int cols, float eps) {
+  __shared__ float red[8];
+  const half_t* x = in + (size_t)blockIdx.x * cols;
+  half_t* y = out + (size_t)blockIdx.x * cols;
+  float s = 0.0f;
+  for (int i = threadIdx.x; i < cols; i += 256) {
+    float v = (float)x[i];
+    s = fmaf(v, v, s);
+  }
+  const float total = block256_sum_ref_order(s, red);
+  const float rms_inv = 1.0f / sqrtf(total / (float)cols + eps);
+  for (int i = threadIdx.x; i < cols; i += 256) {
+    half_t inner = round_f16((float)x[i] * rms_inv);
+    y[i] = round_f16((float)weights[i] * (float)inner);
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
+// rotary, llama_cu.cu:368-389.  One thread per interleaved pair; cos/sin from the host-built
+// table.  real*cos - imag*sin and real*sin + imag*cos each use one fused multiply-add.
+// ---------------------------------------------------------------------------------------------
+__global__ void rope_kernel(half_t* out, const half_t* in, int rows, int cols, int head_dim, int pos_offset,
+                            const float2* __restrict__ table) {
+  const int pair = blockIdx.x * blockDim.x + threadIdx.x;
+  const int r = blockIdx.y;
+  if (pair * 2 >= cols) return;
+  const int c = pair * 2;
+  const float2 cs = table[(size_t)(pos_offset + r) * (head_dim / 2) + (c % head_dim) / 2];
+  const size_t o = (size_t)r * cols + c;
+  const half2_t v = *reinterpret_cast<const half2_t*>(in + o);
+  const float real = (float)v.x, imag = (float)v.y;
+  half2_t w;
+  w.x = round_f16(fmaf(real, cs.x, -(imag * cs.y)));
+  w.y = round_f16(fmaf(real, cs.y, imag * cs.x));
+  *reinterpret_cast<half2_t*>(out + o) = w;
+}
+
+// ---------------------------------------------------------------------------------------------
+// softmax_rows, llama_cu.cu:433-499.  One 256-thread block per row, thread t owns elements
+// t, t+256, ...; the exponential sum is associated as in the reference.
+// ---------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void softmax_rows_kernel(half_t* out, const half_t* in, int w, float temp) {
+  __shared__ float red[8];
+  const half_t* x = in + (size_t)blockIdx.x * w;
+  half_t* y = out + (size_t)blockIdx.x * w;
+  float m = -INFINITY;
+  for (int i = threadIdx.x; i < w; i += 256) {
+    m = fmaxf(m, (float)x[i] / temp);
+  }
+  m = block256_max(m, red);
+  float s = 0.0f;
+  for (int i = threadIdx.x; i < w; i += 256) {
+    s += expf((float)x[i] / temp - m);
+  }
+  const float total = block256_sum_ref_order(s, red);
+  for (int i = threadIdx.x; i < w; i += 256) {
+    y[i] = round_f16(expf((float)x[i] / temp - m) / total);
+  }
+}
+
+// silu, llama_cu.cu:533-539
+__global__ void silu_mul_kernel(half_t* __restrict__ out, const half_t* __restrict__ a, const half_t* __restrict__ b,
+                                size_t size) {
+  const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < size) {
+    const float val = (float)a[i];
+    out[i] = round_f16(val / (1.0f + expf(-val)) * (float)b[i]);
+  }
+}
+
+// embed, llama_cu.cu:32-44: one block per token, 16-byte copies.  An id outside the table gives
+// a zero row instead of a stray read.
+__global__ void embed_kernel(half_t* __restrict__ out, const short* __restrict__ ids, int dim,
+                             const half_t* __restrict__ table, int n_vocab) {
+  const int id = ids[blockIdx.x];
+  const bool ok = id >= 0 && id < n_vocab;
+  const uint4* src = reinterpret_cast<const uint4*>(table + (size_t)(ok ? id : 0) * dim);
+  uint4* dst = reinterpret_cast<uint4*>(out + (size_t)blockIdx.x * dim);
+  for (int i = threadIdx.x; i < dim / 8; i += blockDim.x) {
+    dst[i] = ok ? src[i] : make_uint4(0, 0, 0, 0);
+  }
+}
+
+// embed_uint8, llama_cu.cu:46-62
+__global__ void embed_u8_kernel(half_t* __restrict__ out, const short* __restrict__ ids, int dim,
+                                const uint8_t* __restrict__ codes, const half_t* __restrict__ scales, int block,
+                                int n_vocab) {
+  const int id = ids[blockIdx.x];
+  const bool ok = id >= 0 && id < n_vocab;
+  const int nblk = dim / block;
+  for (int i = threadIdx.x; i < dim; i += blockDim.x) {
+    half_t v = (half_t)0.0f;
+    if (ok) {
+      v = dequant_one(codes[(size_t)id * dim + i], (float)scales[(size_t)id * nblk + i / block]);
+    }
+    out[(size_t)blockIdx.x * dim + i] = v;
+  }
+}
+
+// first maximum of n fp16 values compared as float, llama_cu.cu:1205-1209
+__global__ __launch_bounds__(1024) void argmax_kernel(int* out, const half_t* __restrict__ v, int n) {
+  __shared__ float sval[16];
+  __shared__ int sidx[16];
+  float best = -INFINITY;
+  int idx = 0x7fffffff;
+  for (int i = threadIdx.x; i < n; i += 1024) {
+    const float f = (float)v[i];
+    if (idx == 0x7fffffff || best < f) {  // strict: an equal later value never replaces
+      best = f;
+      idx = i;
+    }
+  }
+  // (value, index) pairs merge by "larger value, then smaller index"; empty slots are (-inf, INT_MAX)
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) {
+    const float ob = __shfl_xor(best, off, WAVE);
+    const int oi = __shfl_xor(idx, off, WAVE);
+    if (ob > best || (ob == best && oi < idx)) {
+      best = ob;
+      idx = oi;
+    }
+  }
+  if ((threadIdx.x & 63) == 0) {
+    sval[threadIdx.x >> 6] = best;
+    sidx[threadIdx.x >> 6] = idx;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int w = 1; w < 16; ++w) {
+      if (sval[w] > best || (sval[w] == best && sidx[w] < idx)) {
+        best = sval[w];
+        idx = sidx[w];
+      }
+    }
+    *out = idx == 0x7fffffff ? 0 : idx;
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
+// quantize_absmax_uint8, transform.cu:28-72.  One wavefront per (row, block of `block` elements).
+// IEEE-only arithmetic: fp32 max, correctly rounded division, round-half-away; the conversion to
+// uint8 saturates and maps NaN (all-zero block: 0/0) to 0.
+// ---------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void quantize_kernel(uint8_t* __restrict__ codes, half_t* __restrict__ scales,
+                                                       const half_t* __restrict__ in, size_t n_blocks, int block) {
+  const size_t b = (size_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (b >= n_blocks) return;
+  const int lane = threadIdx.x & 63;
+  const half_t* src = in + b * block;
+  float absmax = 0.0f;
+  for (int i = lane; i < block; i += WAVE) {
+    absmax = fmaxf(absmax, fabsf((float)src[i]));
+  }
+  absmax = wave_max(absmax);
+  const half_t sh = round_f16(absmax / 127.5f);
+  if (lane == 0) {
+    scales[b] = sh;
+  }
+  const float s = (float)sh;
+  uint8_t* dst = codes + b * block;
+  for (int i = lane; i < block; i += WAVE) {
+    const float v = roundf(127.5f + (float)src[i] / s);
+    dst[i] = (v >= 255.0f) ? (uint8_t)255 : (v > 0.0f ? (uint8_t)v : (uint8_t)0);
+  }
+}
+
+// dequantize_absmax_uint8, transform.cu:74-87: 8 codes per thread
+__global__ void dequantize_kernel(half_t* __restrict__ out, const half_t* __restrict__ scales,
+                                  const uint8_t* __restrict__ codes, size_t n_chunks, int block) {
+  const size_t c = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (c >= n_chunks) return;
+  const uint2 q = *reinterpret_cast<const uint2*>(codes + c * 8);
+  const float s = (float)scales[(c * 8) / block];
+  half8_t r;
+  r[0] = dequant_one(q.x & 0xFF, s);
+  r[1] = dequant_one((q.x >> 8) & 0xFF, s);
+  r[2] = dequant_one((q.x >> 16) & 0xFF, s);
+  r[3] = dequant_one(q.x >> 24, s);
+  r[4] = dequant_one(q.y & 0xFF, s);
+  r[5] = dequant_one((q.y >> 8) & 0xFF, s);
+  r[6] = dequant_one((q.y >> 16) & 0xFF, s);
+  r[7] = dequant_one(q.y >> 24, s);
+  *reinterpret_cast<half8_t*>(out + c * 8) = r;
+}
+
+__device__ __forceinline__ uint64_t splitmix64(uint64_t z) {
+  z += 0x9E3779B97F4A7C15ull;
+  z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+  z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+  return z ^ (z >> 31);
+}
+__device__ __forceinline__ int sum16(uint64_t h) {
+  return int(h & 0xFFFF) + int((h >> 16) & 0xFFFF) + int((h >> 32) & 0xFFFF) + int(h >> 48);
+}
+
+__global__ void fill_normal_kernel(half_t* out, size_t n, uint64_t key, float scale) {
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) {
+    const uint64_t h1 = splitmix64(key + i);
+    const uint64_t h2 = splitmix64(h1);
+    const int s = sum16(h1) + sum16(h2) - 262140;
+    out[i] = round_f16((float)s * scale);
+  }
+}
+
+__global__ void fill_u16_kernel(uint16_t* out, size_t n, uint16_t bits) {
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) {
+    out[i] = bits;
+  }
+}
+
+__global__ void fill_bytes_kernel(uint8_t* out, size_t bytes, uint8_t value) {
+  // 16-byte stores over the aligned middle, single bytes at the ends
+  const size_t tid = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const size_t stride = (size_t)gridDim.x * blockDim.x;
+  const size_t head = ((16 - ((uintptr_t)out & 15)) & 15) < bytes ? ((16 - ((uintptr_t)out & 15)) & 15) : bytes;
+  const size_t n16 = (bytes - head) / 16;
+  const uint32_t w = value * 0x01010101u;
+  uint4* mid = reinterpret_cast<uint4*>(out + head);
+  for (size_t i = tid; i < n16; i += stride) {
+    mid[i] = make_uint4(w, w, w, w);
+  }
+  const size_t tail_start = head + n16 * 16;
+  for (size_t i = tid; i < head; i += stride) out[i] = value;
+  for (size_t i = tail_start + tid; i < bytes; i += stride) out[i] = value;
+}
+
+inline int grid_for(size_t n, int threads, int cap = 1 << 16) {
+  size_t g = (n + threads - 1) / threads;
+  return (int)(g < 1 ? 1 : (g > (size_t)cap ? cap : g));
+}
+
+}  // namespace
+
+extern "C" {
+
+// A fill kernel rather than hipMemsetAsync, so that the call may be recorded into a HIP graph.
+int lcu_memset(void* dev, int byte_value, size_t bytes, void* stream) {
+  if (bytes == 0) return LCU_OK;
+  LCU_REQUIRE(dev != nullptr, "lcu_memset: null pointer");
+  fill_bytes_kernel<<<grid_for(bytes / 16 + 1, 256, 4096), 256, 0, as_stream(stream)>>>((uint8_t*)dev, bytes,
+                                                                                         (uint8_t)byte_value);
+  LCU_LAUNCH_CHECK();
+  return LCU_OK;
+}
+
+int lcu_rmsnorm(void* out_dev, const void* in_dev, const void* weights_dev, int rows, int cols, float eps,
+                void* stream) {
+  LCU_REQUIRE(out_dev && in_dev && weights_dev, "lcu_rmsnorm: null pointer");
+  LCU_REQUIRE(rows >= 0 && cols > 0, "lcu_rmsnorm: bad shape %d x %d", rows, cols);
+  if (rows == 0) return LCU_OK;
+  rmsnorm_kernel<<<rows, 256, 0, as_stream(stream)>>>((half_t*)out_dev, (const half_t*)in_dev,
+                                                      (const half_t*)weights_dev, cols, eps);
+  LCU_LAUNCH_CHECK();
+  return LCU_OK;
+}
+
+int lcu_rope_table_create(void** out_table_dev, int positions, int head_dim, float theta) {
+  LCU_REQUIRE(out_table_dev && positions > 0 && head_dim > 0 && head_dim % 2 == 0,
+              "lcu_rope_table_create: bad arguments (%d positions, head_dim %d)", positions, head_dim);
+  const int half = head_dim / 2;
+  const size_t n = (size_t)positions * half;
+  float2* host = (float2*)malloc(n * sizeof(float2));
+  LCU_REQUIRE(host != nullptr, "lcu_rope_table_create: out of host memory");
+  for (int pos = 0; pos < positions; ++pos) {
+    for (int p = 0; p < half; ++p) {
+      // llama_cu.cu:381: angle = pos / powf(theta, float(c mod head_dim) / head_dim), c = 2p
+      const float angle = (float)pos / powf(theta, (float)(2 * p) / head_dim);
+      host[(size_t)pos * half + p] = make_float2(cosf(angle), sinf(angle));
+    }
+  }
+  void* dev = nullptr;
+  hipError_t e = hipMalloc(&dev, n * sizeof(float2));
+  if (e == hipSuccess) e = hipMemcpy(dev, host, n * sizeof(float2), hipMemcpyHostToDevice);
+  free(host);
+  if (e != hipSuccess) {
+    if (dev) (void)hipFree(dev);
+    return set_error(LCU_E_HIP, "lcu_rope_table_create: %s", hipGetErrorString(e));
+  }
+  *out_table_dev = dev;
+  return LCU_OK;
+}
+
+int lcu_rope(void* out_dev, const void* in_dev, int rows, int cols, int n_heads, int pos_offset,
+             const void* table_dev, int table_positions, void* stream) {
+  LCU_REQUIRE(out_dev && in_dev && table_dev, "lcu_rope: null pointer");
+  LCU_REQUIRE(rows >= 0 && cols > 0 && n_heads > 0 && cols % n_heads == 0 && (cols / n_heads) % 2 == 0,
+              "lcu_rope: bad shape rows %d cols %d heads %d", rows, cols, n_heads);
+  LCU_REQUIRE(pos_offset >= 0 && pos_offset + rows <= table_positions,
+              "lcu_rope: positions %d..%d outside the table of %d", pos_offset, pos_offset + rows, table_positions);
+  if (rows == 0) return LCU_OK;
+  dim3 grid((cols / 2 + 255) / 256, rows);
+  rope_kernel<<<grid, 256, 0, as_stream(stream)>>>((half_t*)out_dev, (const half_t*)in_dev, rows, cols,
+                                                   cols / n_heads, pos_offset, (const float2*)table_dev);
+  LCU_LAUNCH_CHECK();
+  return LCU_OK;
+}
+
+int lcu_softmax_rows(void* out_dev, const void* in_dev, int rows, int w, float temp, void* stream) {
+  LCU_REQUIRE(out_dev && in_dev, "lcu_softmax_rows: null pointer");
+  LCU_REQUIRE(rows >= 0 && w > 0 && temp > 0.0f, "lcu_softmax_rows: bad arguments rows %d w %d temp %f", rows, w,
+              (double)temp);
+  if (rows == 0) return LCU_OK;
+  softmax_rows_kernel<<<rows, 256, 0, as_stream(stream)>>>((half_t*)out_dev, (const half_t*)in_dev, w, temp);
+  LCU_LAUNCH_CHECK();
+  return LCU_OK;
+}
+
+int lcu_silu_mul(void* out_dev, const void* a_dev, const void* b_dev, size_t size, void* stream) {
+  LCU_REQUIRE(out_dev && a_dev && b_dev, "lcu_silu_mul: null pointer");
+  if (size == 0) return LCU_OK;
+  LCU_REQUIRE(size <= ((size_t)1 << 40), "lcu_silu_mul: size too large");
+  silu_mul_kernel<<<(unsigned)((size + 255) / 256), 256, 0, as_stream(stream)>>>(
+      (half_t*)out_dev, (const half_t*)a_dev, (const half_t*)b_dev, size);
+  LCU_LAUNCH_CHECK();
+  return LCU_OK;
+}
+
+int lcu_embed(void* out_dev, const void* ids_dev, int n_ids, int dim, const void* table_dev, int n_vocab,
+              void* stream) {
+  LCU_REQUIRE(out_dev && ids_dev && table_dev, "lcu_embed: null pointer");
+  LCU_REQUIRE(n_ids >= 0 && dim > 0 && dim % 8 == 0 && n_vocab > 0, "lcu_embed: bad shape n %d dim %d", n_ids, dim);
+  if (n_ids == 0) return LCU_OK;
+  embed_kernel<<<n_ids, 256, 0, as_stream(stream)>>>((half_t*)out_dev, (const short*)ids_dev, dim,
+                                                     (const half_t*)table_dev, n_vocab);
+  LCU_LAUNCH_CHECK();
+  return LCU_OK;
+}
+
+int lcu_embed_u8(void* out_dev, const void* ids_dev, int n_ids, int dim, const void* codes_dev,
+                 const void* scales_dev, int block, int n_vocab, void* stream) {
+  LCU_REQUIRE(out_dev && ids_dev && codes_dev && scales_dev, "lcu_embed_u8: null pointer");
+  LCU_REQUIRE(n_ids >= 0 && dim > 0 && block > 0 && dim % block == 0 && n_vocab > 0,
+              "lcu_embed_u8: bad shape n %d dim %d block %d", n_ids, dim, block);
+  if (n_ids == 0) return LCU_OK;
+  embed_u8_kernel<<<n_ids, 256, 0, as_stream(stream)>>>((half_t*)out_dev, (const short*)ids_dev, dim,
+                                                        (const uint8_t*)codes_dev, (const half_t*)scales_dev, block,
+                                                        n_vocab);
+  LCU_LAUNCH_CHECK();
+  return LCU_OK;
+}
+
+int lcu_argmax_f16(void* out_index_dev, const void* values_dev, int n, void* stream) {
+  LCU_REQUIRE(out_index_dev && values_dev && n > 0, "lcu_argmax_f16: bad arguments");
+  argmax_kernel<<<1, 1024, 0, as_stream(stream)>>>((int*)out_index_dev, (const half_t*)values_dev, n);
+  LCU_LAUNCH_CHECK();
+  return LCU_OK;
+}
+
+int lcu_quantize_absmax_u8(void* codes_dev, void* scales_dev, const void* in_dev, size_t rows, size_t cols,
+                           int block, void* stream) {
+  LCU_REQUIRE(codes_dev && scales_dev && in_dev, "lcu_quantize_absmax_u8: null pointer");
+  LCU_REQUIRE(block > 0 && cols % block == 0, "lcu_quantize_absmax_u8: cols %zu not a multiple of block %d", cols,
+              block);
+  const size_t n_blocks = rows * (cols / block);
+  if (n_blocks == 0) return LCU_OK;
+  LCU_REQUIRE((n_blocks + 3) / 4 < ((size_t)1 << 31), "lcu_quantize_absmax_u8: tensor too large");
+  quantize_kernel<<<(unsigned)((n_blocks + 3) / 4), 256, 0, as_stream(stream)>>>(
+      (uint8_t*)codes_dev, (half_t*)scales_dev, (const half_t*)in_dev, n_blocks, block);
+  LCU_LAUNCH_CHECK();
+  return LCU_OK;
+}
+
+int lcu_dequantize_absmax_u8(void* out_dev, const void* scales_dev, const void* codes_dev, size_t rows,
+                             size_t cols, int block, void* stream) {
+  LCU_REQUIRE(out_dev && scales_dev && codes_dev, "lcu_dequantize_absmax_u8: null pointer");
+  LCU_REQUIRE(block > 0 && block % 8 == 0 && cols % block == 0,
+              "lcu_dequantize_absmax_u8: cols %zu / block %d unsupported (block must be a multiple of 8)", cols, block);
+  const size_t n_chunks = rows * cols / 8;
+  if (n_chunks == 0) return LCU_OK;
+  LCU_REQUIRE((n_chunks + 255) / 256 < ((size_t)1 << 31), "lcu_dequantize_absmax_u8: tensor too large");
+  dequantize_kernel<<<(unsigned)((n_chunks + 255) / 256), 256, 0, as_stream(stream)>>>(
+      (half_t*)out_dev, (const half_t*)scales_dev, (const uint8_t*)codes_dev, n_chunks, block);
+  LCU_LAUNCH_CHECK();
+  return LCU_OK;
+}
+
+int lcu_fill_normal_f16(void* out_dev, size_t n, uint64_t seed, uint64_t stream_id, float std, void* stream) {
+  LCU_REQUIRE(out_dev || n == 0, "lcu_fill_normal_f16: null pointer");
+  if (n == 0) return LCU_OK;
+  uint64_t z = seed ^ (stream_id * 0xD1B54A32D192ED03ull);
+  z += 0x9E3779B97F4A7C15ull;
+  z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+  z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+  const uint64_t key = z ^ (z >> 31);
+  const double sigma = sqrt(8.0 * (65536.0 * 65536.0 - 1.0) / 12.0);
+  const float scale = (float)((double)std / sigma);
+  fill_normal_kernel<<<grid_for(n, 256, 8192), 256, 0, as_stream(stream)>>>((half_t*)out_dev, n, key, scale);
+  LCU_LAUNCH_CHECK();
+  return LCU_OK;
+}
+
+int lcu_fill_f16(void* out_dev, size_t n, uint16_t bits, void* stream) {
+  LCU_REQUIRE(out_dev || n == 0, "lcu_fill_f16: null pointer");
+  if (n == 0) return LCU_OK;
+  fill_u16_kernel<<<grid_for(n, 256, 4096), 256, 0, as_stream(stream)>>>((uint16_t*)out_dev, n, bits);
+  LCU_LAUNCH_CHECK();
+  return LCU_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,188 @@
+// Runtime part of the C ABI: device set-up, buffers, copies, streams, events.
+// Counterpart of llama_cu.cu:691-736 (scoped_gpu, gpu_buffer, gpu_buffer_view) and 1525-1542
+// (initialize) in the reference.
+#include <stdarg.h>
+#include <string.h>
+
+#include "common.hpp"
+
+namespace lcu {
+
+static thread_local char g_error[512] = "";
+static device_state g_devices[16];
+
+int set_error(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_error, sizeof(g_error), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+device_state* current_device_state() {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 16) {
+    return nullptr;
+  }
+  return &g_devices[dev];
+}
+
+}  // namespace lcu
+
+using namespace lcu;
+
+extern "C" {
+
+const char* lcu_last_error(void) { return g_error; }
+
+int lcu_init(int device) {
+  LCU_REQUIRE(device >= 0 && device < 16, "lcu_init: device %d out of range", device);
+  LCU_HIP(hipSetDevice(device));
+  device_state& st = g_devices[device];
+  if (st.ready) {
+    return LCU_OK;
+  }
+  hipDeviceProp_t prop;
+  LCU_HIP(hipGetDeviceProperties(&prop, device));
+  if (strncmp(prop.gcnArchName, "gfx950", 6) != 0) {
+    return set_error(LCU_E_HIP, "lcu_init: device %d is %s, this library is built for gfx950 only",
+                     device, prop.gcnArchName);
+  }
+  st.compute_units = prop.multiProcessorCount;
+  // attention workspace: partial outputs of up to 64 heads x 32 splits x (128 + 2) floats,
+  // followed by one arrival counter per head
+  st.workspace_bytes = 4u << 20;
+  LCU_HIP(hipMalloc(&st.workspace, st.workspace_bytes));
+  LCU_HIP(hipMemset(st.workspace, 0, st.workspace_bytes));
+  LCU_HIP(hipDeviceSynchronize());
+  st.ready = true;
+  return LCU_OK;
+}
+
+int lcu_device_get_props(int device, lcu_device_props* out) {
+  LCU_REQUIRE(out != nullptr, "lcu_device_get_props: null output");
+  hipDeviceProp_t prop;
+  LCU_HIP(hipGetDeviceProperties(&prop, device));
+  memset(out, 0, sizeof(*out));
+  snprintf(out->name, sizeof(out->name), "%s (%s)", prop.name, prop.gcnArchName);
+  out->compute_units = prop.multiProcessorCount;
+  out->lds_bytes_per_block = (int)prop.sharedMemPerBlock;
+  out->l2_bytes = prop.l2CacheSize;
+  out->clock_khz = prop.clockRate;
+  out->memory_clock_khz = prop.memoryClockRate;
+  out->memory_bus_bits = prop.memoryBusWidth;
+  out->total_memory = prop.totalGlobalMem;
+  size_t free_b = 0, total_b = 0;
+  int prev = 0;
+  LCU_HIP(hipGetDevice(&prev));
+  LCU_HIP(hipSetDevice(device));
+  LCU_HIP(hipMemGetInfo(&free_b, &total_b));
+  LCU_HIP(hipSetDevice(prev));
+  out->free_memory = free_b;
+  return LCU_OK;
+}
+
+int lcu_get_device(int* out_device) {
+  LCU_REQUIRE(out_device != nullptr, "lcu_get_device: null output");
+  LCU_HIP(hipGetDevice(out_device));
+  return LCU_OK;
+}
+
+int lcu_set_device(int device) {
+  LCU_HIP(hipSetDevice(device));
+  return LCU_OK;
+}
+
+int lcu_malloc(void** out_dev, size_t bytes) {
+  LCU_REQUIRE(out_dev != nullptr, "lcu_malloc: null output");
+  *out_dev = nullptr;
+  if (bytes == 0) {
+    return LCU_OK;
+  }
+  LCU_HIP(hipMalloc(out_dev, bytes));
+  return LCU_OK;
+}
+
+int lcu_free(void* dev) {
+  if (dev) {
+    LCU_HIP(hipFree(dev));
+  }
+  return LCU_OK;
+}
+
+int lcu_h2d(void* dst_dev, const void* src_host, size_t bytes, void* stream) {
+  if (bytes == 0) return LCU_OK;
+  LCU_REQUIRE(dst_dev && src_host, "lcu_h2d: null pointer");
+  LCU_HIP(hipMemcpyAsync(dst_dev, src_host, bytes, hipMemcpyHostToDevice, as_stream(stream)));
+  return LCU_OK;
+}
+
+int lcu_d2h(void* dst_host, const void* src_dev, size_t bytes, void* stream) {
+  if (bytes == 0) return LCU_OK;
+  LCU_REQUIRE(dst_host && src_dev, "lcu_d2h: null pointer");
+  LCU_HIP(hipMemcpyAsync(dst_host, src_dev, bytes, hipMemcpyDeviceToHost, as_stream(stream)));
+  LCU_HIP(hipStreamSynchronize(as_stream(stream)));
+  return LCU_OK;
+}
+
+int lcu_d2d(void* dst_dev, const void* src_dev, size_t bytes, void* stream) {
+  if (bytes == 0) return LCU_OK;
+  LCU_REQUIRE(dst_dev && src_dev, "lcu_d2d: null pointer");
+  LCU_HIP(hipMemcpyAsync(dst_dev, src_dev, bytes, hipMemcpyDeviceToDevice, as_stream(stream)));
+  return LCU_OK;
+}
+
+int lcu_stream_create(void** out_stream) {
+  LCU_REQUIRE(out_stream != nullptr, "lcu_stream_create: null output");
+  hipStream_t s;
+  LCU_HIP(hipStreamCreateWithFlags(&s, hipStreamNonBlocking));  // default priority
+  *out_stream = s;
+  return LCU_OK;
+}
+
+int lcu_stream_destroy(void* stream) {
+  if (stream) {
+    LCU_HIP(hipStreamDestroy(as_stream(stream)));
+  }
+  return LCU_OK;
+}
+
+int lcu_sync(void* stream) {
+  if (stream) {
+    LCU_HIP(hipStreamSynchronize(as_stream(stream)));
+  } else {
+    LCU_HIP(hipDeviceSynchronize());
+  }
+  return LCU_OK;
+}
+
+int lcu_event_create(void** out_event) {
+  LCU_REQUIRE(out_event != nullptr, "lcu_event_create: null output");
+  hipEvent_t e;
+  LCU_HIP(hipEventCreate(&e));
+  *out_event = e;
+  return LCU_OK;
+}
+
+int lcu_event_destroy(void* event) {
+  if (event) {
+    LCU_HIP(hipEventDestroy(reinterpret_cast<hipEvent_t>(event)));
+  }
+  return LCU_OK;
+}
+
+int lcu_event_record(void* event, void* stream) {
+  LCU_REQUIRE(event != nullptr, "lcu_event_record: null event");
+  LCU_HIP(hipEventRecord(reinterpret_cast<hipEvent_t>(event), as_stream(stream)));
+  return LCU_OK;
+}
+
+int lcu_event_elapsed_ms(float* out_ms, void* start_event, void* stop_event) {
+  LCU_REQUIRE(out_ms && start_event && stop_event, "lcu_event_elapsed_ms: null argument");
+  LCU_HIP(hipEventSynchronize(reinterpret_cast<hipEvent_t>(stop_event)));
+  LCU_HIP(hipEventElapsedTime(out_ms, reinterpret_cast<hipEvent_t>(start_event),
+                              reinterpret_cast<hipEvent_t>(stop_event)));
+  return LCU_OK;
+}
+
+}  // extern "C"

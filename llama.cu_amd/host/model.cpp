@@ -1,0 +1,366 @@
+// Model weights and the forward pass: the host orchestration of llama_cu.cu:882-1310
+// (llama_layer, llama_model_impl, llama_context_impl) over the C ABI of llama_cu_hip.h.
+//
+// What is kept from the reference: the order of operations of next_token, every point where an
+// intermediate is rounded to fp16, the [position][dim] KV cache, the per-tensor file format, the
+// first-maximum argmax over the fp16 probabilities.  What is not: its zeroed gutter rows, its
+// per-layer score-tensor allocation, its side streams, its re-rotation of every cached K row on
+// every call (K is cached rotated; RoPE depends only on value and position, so the bits agree),
+// and its one-launch-per-operation decode loop (a single new token runs the fused kernels).
+#include <assert.h>
+#include <string.h>
+
+#include "model_impl.hpp"
+
+namespace llama_cu {
+
+namespace {
+
+constexpr uint16_t FP16_ONE = 0x3C00;
+
+bool load_matrix(weight_tensor& t, llama_params const& params, std::string const& path, std::string const& name,
+                 size_t h, size_t w) {
+  // llama_cu.cu:929-971: <name>.weight__<h>_<w> holds fp16 values or uint8 codes,
+  // <name>.scale__<h>_<w/block> the fp16 scales of a quantised tensor
+  t.rows = h;
+  t.cols = w;
+  const std::string stem = path + "/" + name;
+  if (params.q_type == quantization_type::fp16) {
+    t.quantised = false;
+    t.block = 0;
+    t.data = gpu_buffer(h * w * 2);
+    mapped_buffer buf(stem + ".weight__" + std::to_string(h) + "_" + std::to_string(w));
+    if (!buf.is_ok() || buf.size() != t.data.size()) {
+      fprintf(stderr, "failed to load tensor %s (%zu x %zu)\n", name.c_str(), h, w);
+      return false;
+    }
+    t.data.copy_from(buf);
+    LCU_CHECK(lcu_sync(nullptr));  // the mapping goes away at the end of this scope
+    return true;
+  }
+  if (params.q_type == quantization_type::uint8) {
+    const size_t block = params.quantization_block_size;
+    if (block == 0 || w % block != 0) {
+      fprintf(stderr, "failed to load tensor %s: width %zu is not a multiple of block %zu\n", name.c_str(), w, block);
+      return false;
+    }
+    t.quantised = true;
+    t.block = (int)block;
+    t.data = gpu_buffer(h * w);
+    t.scales = gpu_buffer(h * (w / block) * 2);
+    mapped_buffer wbuf(stem + ".weight__" + std::to_string(h) + "_" + std::to_string(w));
+    if (!wbuf.is_ok() || wbuf.size() != t.data.size()) {
+      fprintf(stderr, "failed to load tensor %s (%zu x %zu)\n", name.c_str(), h, w);
+      return false;
+    }
+    t.data.copy_from(wbuf);
+    mapped_buffer sbuf(stem + ".scale__" + std::to_string(h) + "_" + std::to_string(w / block));
+    if (!sbuf.is_ok() || sbuf.size() != t.scales.size()) {
+      fprintf(stderr, "failed to load tensor scale %s (%zu x %zu)\n", name.c_str(), h, w / block);
+      return false;
+    }
+    t.scales.copy_from(sbuf);
+    LCU_CHECK(lcu_sync(nullptr));
+    return true;
+  }
+  fprintf(stderr, "Unsupported quantization type %d\n", (int)params.q_type);
+  return false;
+}
+
+bool load_vector(gpu_buffer& t, std::string const& path, std::string const& name, size_t w) {
+  // llama_cu.cu:972-984
+  t = gpu_buffer(w * 2);
+  mapped_buffer buf(path + "/" + name + ".weight__" + std::to_string(w));
+  if (!buf.is_ok() || buf.size() != t.size()) {
+    fprintf(stderr, "failed to load tensor %s\n", name.c_str());
+    return false;
+  }
+  t.copy_from(buf);
+  LCU_CHECK(lcu_sync(nullptr));
+  return true;
+}
+
+void synth_matrix(weight_tensor& t, llama_params const& params, gpu_buffer& staging, size_t h, size_t w, uint64_t seed,
+                  uint64_t stream_id, float std) {
+  t.rows = h;
+  t.cols = w;
+  if (params.q_type == quantization_type::uint8) {
+    const int block = params.quantization_block_size;
+    t.quantised = true;
+    t.block = block;
+    t.data = gpu_buffer(h * w);
+    t.scales = gpu_buffer(h * (w / block) * 2);
+    if (staging.size() < h * w * 2) {
+      staging = gpu_buffer();  // release before growing
+      staging = gpu_buffer(h * w * 2);
+    }
+    LCU_CHECK(lcu_fill_normal_f16(staging.data(), h * w, seed, stream_id, std, nullptr));
+    LCU_CHECK(lcu_quantize_absmax_u8(t.data.data(), t.scales.data(), staging.data(), h, w, block, nullptr));
+  } else {
+    t.quantised = false;
+    t.block = 0;
+    t.data = gpu_buffer(h * w * 2);
+    LCU_CHECK(lcu_fill_normal_f16(t.data.data(), h * w, seed, stream_id, std, nullptr));
+  }
+}
+
+void synth_ones(gpu_buffer& t, size_t w) {
+  t = gpu_buffer(w * 2);
+  LCU_CHECK(lcu_fill_f16(t.data(), w, FP16_ONE, nullptr));
+}
+
+}  // namespace
+
+bool llama_model_impl::load_impl(std::string const& path) {
+  // llama_cu.cu:891-922
+  const size_t dim = params.dim, ffn = params.ffn_dim(), vocab = params.n_vocab;
+  RETURN_UNLESS(load_matrix(tok_embeddings, params, path, "tok_embeddings", vocab, dim));
+  RETURN_UNLESS(load_matrix(output, params, path, "output", vocab, dim));
+  RETURN_UNLESS(load_vector(norm, path, "norm", dim));
+  layers.clear();
+  layers.reserve(params.n_layers);
+  for (uint32_t i = 0; i < params.n_layers; ++i) {
+    llama_layer L;
+    const std::string base = "layers." + std::to_string(i) + ".";
+    RETURN_UNLESS(load_vector(L.attn_norm, path, base + "attention_norm", dim));
+    RETURN_UNLESS(load_vector(L.ffn_norm, path, base + "ffn_norm", dim));
+    RETURN_UNLESS(load_matrix(L.wq, params, path, base + "attention.wq", dim, dim));
+    RETURN_UNLESS(load_matrix(L.wk, params, path, base + "attention.wk", dim, dim));
+    RETURN_UNLESS(load_matrix(L.wv, params, path, base + "attention.wv", dim, dim));
+    RETURN_UNLESS(load_matrix(L.wo, params, path, base + "attention.wo", dim, dim));
+    RETURN_UNLESS(load_matrix(L.w1, params, path, base + "feed_forward.w1", ffn, dim));
+    RETURN_UNLESS(load_matrix(L.w2, params, path, base + "feed_forward.w2", dim, ffn));
+    RETURN_UNLESS(load_matrix(L.w3, params, path, base + "feed_forward.w3", ffn, dim));
+    layers.emplace_back(std::move(L));
+  }
+  return true;
+}
+
+void llama_model_impl::synthesize(uint64_t seed, float std) {
+  const size_t dim = params.dim, ffn = params.ffn_dim(), vocab = params.n_vocab;
+  gpu_buffer staging;
+  synth_matrix(tok_embeddings, params, staging, vocab, dim, seed, 1, std);
+  synth_matrix(output, params, staging, vocab, dim, seed, 2, std);
+  synth_ones(norm, dim);
+  layers.clear();
+  layers.reserve(params.n_layers);
+  for (uint32_t i = 0; i < params.n_layers; ++i) {
+    llama_layer L;
+    const uint64_t base = 16 + 16 * (uint64_t)i;
+    synth_matrix(L.wq, params, staging, dim, dim, seed, base + 0, std);
+    synth_matrix(L.wk, params, staging, dim, dim, seed, base + 1, std);
+    synth_matrix(L.wv, params, staging, dim, dim, seed, base + 2, std);
+    synth_matrix(L.wo, params, staging, dim, dim, seed, base + 3, std);
+    synth_matrix(L.w1, params, staging, ffn, dim, seed, base + 4, std);
+    synth_matrix(L.w2, params, staging, dim, ffn, seed, base + 5, std);
+    synth_matrix(L.w3, params, staging, ffn, dim, seed, base + 6, std);
+    synth_ones(L.attn_norm, dim);
+    synth_ones(L.ffn_norm, dim);
+    layers.emplace_back(std::move(L));
+  }
+  LCU_CHECK(lcu_sync(nullptr));
+}
+
+weight_tensor const* llama_model_impl::tensor_by_stream(uint64_t stream_id) const {
+  if (stream_id == 1) return &tok_embeddings;
+  if (stream_id == 2) return &output;
+  if (stream_id < 16) return nullptr;
+  const size_t l = (stream_id - 16) / 16, which = (stream_id - 16) % 16;
+  if (l >= layers.size() || which > 6) return nullptr;
+  llama_layer const& L = layers[l];
+  weight_tensor const* tab[7] = {&L.wq, &L.wk, &L.wv, &L.wo, &L.w1, &L.w2, &L.w3};
+  return tab[which];
+}
+
+static bool shapes_supported(llama_params const& p) {
+  if (p.n_heads == 0 || p.dim == 0 || p.dim % p.n_heads != 0 || p.dim / p.n_heads != 128) {
+    fprintf(stderr, "unsupported model shape: dim %u with %u heads (head_dim must be 128)\n", p.dim, p.n_heads);
+    return false;
+  }
+  if (p.n_vocab == 0 || p.n_vocab > 32767) {
+    fprintf(stderr, "unsupported vocabulary size %u (token ids are 16-bit)\n", p.n_vocab);
+    return false;
+  }
+  if (p.q_type == quantization_type::uint8) {
+    const uint32_t b = p.quantization_block_size;
+    if (b < 16 || b % 16 != 0 || p.dim % b != 0 || p.ffn_dim() % b != 0) {
+      fprintf(stderr, "unsupported quantization block size %u for dim %u / ffn %u\n", b, p.dim, p.ffn_dim());
+      return false;
+    }
+  } else if (p.q_type != quantization_type::fp16) {
+    fprintf(stderr, "Unsupported quantization type %d\n", (int)p.q_type);
+    return false;
+  }
+  return true;
+}
+
+/* static */ std::unique_ptr<llama_model> llama_model::load(llama_params params, llama_partition partition,
+                                                            std::string const& path) {
+  // llama_cu.cu:987-997
+  if (!shapes_supported(params)) {
+    return nullptr;
+  }
+  auto model = std::make_unique<llama_model_impl>(params, partition);
+  if (!model->load_impl(path)) {
+    return nullptr;
+  }
+  return model;
+}
+
+/* static */ std::unique_ptr<llama_model> llama_model::create_synthetic(llama_params params, uint64_t seed,
+                                                                        float weight_std) {
+  params.magic = LLAMA_CU_MAGIC;
+  params.fourcc = LLAMA_CU_MODEL_FOURCC_LLAMA;
+  if (!shapes_supported(params)) {
+    return nullptr;
+  }
+  llama_partition partition;
+  partition.use_default(params);
+  auto model = std::make_unique<llama_model_impl>(params, partition);
+  model->synthesize(seed, weight_std);
+  return model;
+}
+
+// ------------------------------------------------------------------------------------------------
+// context
+// ------------------------------------------------------------------------------------------------
+llama_context_impl::llama_context_impl(llama_model* model, int context_len, float temperature)
+    : llama_context(static_cast<llama_model_impl*>(model), context_len, temperature) {
+  LCU_CHECK(lcu_init(0));
+  LCU_CHECK(lcu_stream_create(&stream_));
+  const int head_dim = model_->params.dim / model_->params.n_heads;
+  LCU_CHECK(lcu_rope_table_create(&rope_table_, context_len_, head_dim, 10000.0f));  // theta: llama_cu.cu:374
+  clear_tokens();
+}
+
+llama_context_impl::~llama_context_impl() {
+  lcu_sync(stream_);
+  lcu_free(rope_table_);
+  lcu_stream_destroy(stream_);
+}
+
+void llama_context_impl::clear_tokens() {
+  // llama_cu.cu:1004-1049: fresh zeroed KV cache and scratch, position 0
+  llama_params const& p = model_->params;
+  const size_t ctx = (size_t)context_len_, dim = p.dim, ffn = p.ffn_dim();
+  LCU_CHECK(lcu_sync(stream_));
+  kv_.clear();
+  kv_.resize(p.n_layers);
+  for (auto& kv : kv_) {
+    kv.k = gpu_buffer(ctx * dim * 2);
+    kv.v = gpu_buffer(ctx * dim * 2);
+    LCU_CHECK(lcu_memset(kv.k.data(), 0, kv.k.size(), stream_));
+    LCU_CHECK(lcu_memset(kv.v.data(), 0, kv.v.size(), stream_));
+  }
+  if (!t_embed_.is_ok()) {
+    t_embed_ = gpu_buffer(ctx * dim * 2);
+    t_norm_ = gpu_buffer(ctx * dim * 2);
+    t_xq_ = gpu_buffer(ctx * dim * 2);
+    t_out_ = gpu_buffer(ctx * dim * 2);
+    t_w1_ = gpu_buffer(ctx * ffn * 2);
+    t_w3_ = gpu_buffer(ctx * ffn * 2);
+    t_silu_ = gpu_buffer(ctx * ffn * 2);
+    t_tokens_ = gpu_buffer(ctx * sizeof(short));
+    t_logits_ = gpu_buffer((size_t)p.n_vocab * 2);
+    t_probs_ = gpu_buffer((size_t)p.n_vocab * 2);
+    t_argmax_ = gpu_buffer(sizeof(int));
+  }
+  LCU_CHECK(lcu_sync(stream_));
+  start_pos_ = 0;
+  last_n_ = 0;
+}
+
+size_t llama_context_impl::context_memory_usage() {
+  size_t count = 0;
+  for (auto& kv : kv_) {
+    count += kv.k.size() + kv.v.size();
+  }
+  for (gpu_buffer const* b : {&t_embed_, &t_norm_, &t_xq_, &t_out_, &t_w1_, &t_w3_, &t_silu_, &t_tokens_, &t_logits_,
+                              &t_probs_, &t_argmax_}) {
+    count += b->size();
+  }
+  return count;
+}
+
+void llama_context_impl::matmul(void* out, const void* lhs, weight_tensor const& w, int M, float beta) {
+  // llama_cu.cu:1498-1523
+  if (w.quantised) {
+    LCU_CHECK(lcu_gemm_f16u8_nt(out, lhs, w.data.data(), w.scales.data(), M, (int)w.cols, (int)w.rows, w.block, beta,
+                                stream_));
+  } else {
+    LCU_CHECK(lcu_gemm_f16_nt(out, lhs, w.data.data(), M, (int)w.cols, (int)w.rows, beta, stream_));
+  }
+}
+
+short llama_context_impl::next_token(std::vector<short> const& new_tokens) {
+  llama_params const& p = model_->params;
+  const int n = (int)new_tokens.size();
+  assert(n > 0);
+  assert(new_tokens.size() + start_pos_ <= (size_t)context_len_);  // llama_cu.cu:1074
+  const int dim = p.dim, ffn = p.ffn_dim(), heads = p.n_heads, vocab = p.n_vocab;
+  const int sp = start_pos_, T = sp + n;
+  const int block = p.q_type == quantization_type::uint8 ? p.quantization_block_size : 0;
+  char* x = (char*)t_embed_.data();
+
+  // 1086-1097
+  LCU_CHECK(lcu_h2d(t_tokens_.data(), new_tokens.data(), n * sizeof(short), stream_));
+  if (model_->tok_embeddings.quantised) {
+    LCU_CHECK(lcu_embed_u8(x, t_tokens_.data(), n, dim, model_->tok_embeddings.data.data(),
+                           model_->tok_embeddings.scales.data(), block, vocab, stream_));
+  } else {
+    LCU_CHECK(lcu_embed(x, t_tokens_.data(), n, dim, model_->tok_embeddings.data.data(), vocab, stream_));
+  }
+
+  for (size_t l = 0; l < model_->layers.size(); ++l) {
+    llama_layer const& L = model_->layers[l];
+    char* kc = (char*)kv_[l].k.data();
+    char* vc = (char*)kv_[l].v.data();
+    char* k_new = kc + (size_t)sp * dim * 2;
+    char* v_new = vc + (size_t)sp * dim * 2;
+    if (n == 1) {
+      // 1129-1156 in one launch
+      LCU_CHECK(lcu_decode_qkv(t_xq_.data(), kc, vc, x, L.attn_norm.data(), L.wq.data.data(), L.wk.data.data(),
+                               L.wv.data.data(), L.wq.scales.data(), L.wk.scales.data(), L.wv.scales.data(), block, dim,
+                               heads, sp, p.norm_eps, rope_table_, context_len_, stream_));
+    } else {
+      LCU_CHECK(lcu_rmsnorm(t_norm_.data(), x, L.attn_norm.data(), n, dim, p.norm_eps, stream_));            // 1129
+      matmul(t_xq_.data(), t_norm_.data(), L.wq, n, 0.0f);                                                   // 1144
+      LCU_CHECK(lcu_rope(t_xq_.data(), t_xq_.data(), n, dim, heads, sp, rope_table_, context_len_, stream_));  // 1146
+      matmul(k_new, t_norm_.data(), L.wk, n, 0.0f);                                                          // 1150
+      LCU_CHECK(lcu_rope(k_new, k_new, n, dim, heads, sp, rope_table_, context_len_, stream_));  // 1152, new rows only
+      matmul(v_new, t_norm_.data(), L.wv, n, 0.0f);                                                          // 1156
+    }
+    LCU_CHECK(lcu_attention(t_out_.data(), t_xq_.data(), kc, vc, n, T, sp, dim, heads, stream_));            // 1161-1171
+    matmul(x, t_out_.data(), L.wo, n, 1.0f);                                                                 // 1174
+    if (n == 1) {
+      // 1176-1183 in one launch
+      LCU_CHECK(lcu_decode_ffn_up(t_silu_.data(), x, L.ffn_norm.data(), L.w1.data.data(), L.w3.data.data(),
+                                  L.w1.scales.data(), L.w3.scales.data(), block, dim, ffn, p.norm_eps, stream_));
+    } else {
+      LCU_CHECK(lcu_rmsnorm(t_norm_.data(), x, L.ffn_norm.data(), n, dim, p.norm_eps, stream_));             // 1176
+      matmul(t_w1_.data(), t_norm_.data(), L.w1, n, 0.0f);                                                   // 1180
+      matmul(t_w3_.data(), t_norm_.data(), L.w3, n, 0.0f);                                                   // 1181
+      LCU_CHECK(lcu_silu_mul(t_silu_.data(), t_w1_.data(), t_w3_.data(), (size_t)n * ffn, stream_));         // 1183
+    }
+    matmul(x, t_silu_.data(), L.w2, n, 1.0f);                                                                // 1185
+  }
+  // 1191-1197: the reference normalises every row and uses the last one
+  LCU_CHECK(lcu_decode_logits(t_logits_.data(), x + (size_t)(n - 1) * dim * 2, model_->norm.data(),
+                              model_->output.data.data(), model_->output.scales.data(), block, dim, vocab, p.norm_eps,
+                              stream_));
+  LCU_CHECK(lcu_softmax_rows(t_probs_.data(), t_logits_.data(), 1, vocab, temperature_, stream_));
+  // 1198-1209: first maximum of the fp16 probabilities, found on the device; 4 bytes come back
+  LCU_CHECK(lcu_argmax_f16(t_argmax_.data(), t_probs_.data(), vocab, stream_));
+  int token = 0;
+  LCU_CHECK(lcu_d2h(&token, t_argmax_.data(), sizeof(int), stream_));
+  start_pos_ += n;
+  last_n_ = n;
+  return (short)token;
+}
+
+/* static */ std::unique_ptr<llama_context> llama_context::create(llama_model* model, int context_len,
+                                                                  float temperature) {
+  return std::make_unique<llama_context_impl>(model, context_len, temperature);
+}
+
+}  // namespace llama_cu

@@ -1,0 +1,70 @@
+// Implementation types behind llama_model / llama_context (the reference keeps its counterparts,
+// llama_layer / llama_model_impl / llama_context_impl, private to llama_cu.cu:882-1304).
+#pragma once
+#include <string>
+#include <vector>
+
+#include "host_common.hpp"
+
+namespace llama_cu {
+
+// one weight matrix [rows, cols]: fp16 values, or uint8 codes with fp16 scales [rows, cols/block]
+// (the reference's generic_tensor, llama_cu.h:252-270)
+struct weight_tensor {
+  gpu_buffer data;
+  gpu_buffer scales;
+  size_t rows{0}, cols{0};
+  bool quantised{false};
+  int block{0};
+};
+
+struct llama_layer {
+  weight_tensor wq, wk, wv, wo;
+  weight_tensor w1, w2, w3;
+  gpu_buffer attn_norm, ffn_norm;
+};
+
+struct llama_model_impl : public llama_model {
+  llama_model_impl(llama_params params, llama_partition partition) : llama_model(params, partition) {}
+  bool load_impl(std::string const& path);
+  void synthesize(uint64_t seed, float weight_std);
+  weight_tensor const* tensor_by_stream(uint64_t stream_id) const;
+  weight_tensor tok_embeddings;
+  weight_tensor output;
+  gpu_buffer norm;
+  std::vector<llama_layer> layers;
+};
+
+struct llama_context_impl final : public llama_context {
+  llama_context_impl(llama_model* model, int context_len, float temperature);
+  ~llama_context_impl() override;
+  void clear_tokens() override;
+  size_t context_memory_usage() override;
+  short next_token(std::vector<short> const& new_tokens) override;
+
+  // read-back used by tests and tools
+  llama_model_impl* model() const { return model_; }
+  int context_len() const { return context_len_; }
+  int start_pos() const { return start_pos_; }
+  int last_n() const { return last_n_; }
+  void* stream() const { return stream_; }
+  gpu_buffer& hidden() { return t_embed_; }
+  gpu_buffer& logits() { return t_logits_; }
+  gpu_buffer& probs() { return t_probs_; }
+  struct kv_cache_layer {
+    gpu_buffer k;  // [context_len][dim], rotated
+    gpu_buffer v;
+  };
+  std::vector<kv_cache_layer>& kv() { return kv_; }
+
+ private:
+  void matmul(void* out, const void* lhs, weight_tensor const& w, int M, float beta);
+  std::vector<kv_cache_layer> kv_;
+  gpu_buffer t_embed_, t_norm_, t_xq_, t_out_, t_w1_, t_w3_, t_silu_;
+  gpu_buffer t_tokens_, t_logits_, t_probs_, t_argmax_;
+  void* stream_{nullptr};
+  void* rope_table_{nullptr};
+  int last_n_{0};
+};
+
+}  // namespace llama_cu

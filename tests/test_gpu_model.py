@@ -1,0 +1,188 @@
+"""GPU parity of the whole forward pass (llama_context::next_token through the C handles) against
+the CPU oracle: synthetic weights bit-identical, hidden state / logits / probabilities within
+max-abs-rel 1e-2, KV cache contents, greedy tokens."""
+import json
+import os
+
+import numpy as np
+import pytest
+
+import oracle_lib as O
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-2
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+
+
+@pytest.fixture(scope="module", autouse=True)
+def gpu():
+    import gpu_helpers as G
+    G.setup()
+    yield G
+    G.release()
+
+
+TINY = dict(dim=256, multiple_of=128, n_heads=2, n_layers=2, n_vocab=320)
+SMALL = dict(dim=512, multiple_of=128, n_heads=4, n_layers=4, n_vocab=2048)
+
+
+def streams(n_layers):
+    yield 1, "vocab"
+    yield 2, "vocab"
+    for l in range(n_layers):
+        for w in range(7):
+            yield 16 + 16 * l + w, w
+
+
+def shape_of(cfg, ffn, kind):
+    if kind == "vocab":
+        return cfg["n_vocab"], cfg["dim"]
+    return {0: (cfg["dim"], cfg["dim"]), 1: (cfg["dim"], cfg["dim"]), 2: (cfg["dim"], cfg["dim"]),
+            3: (cfg["dim"], cfg["dim"]), 4: (ffn, cfg["dim"]), 5: (cfg["dim"], ffn), 6: (ffn, cfg["dim"])}[kind]
+
+
+@pytest.mark.parametrize("q_type", [0, 1])
+def test_synthetic_weights_bit_identical(gpu, q_type):
+    G = gpu
+    om = O.Model(**TINY, q_type=q_type, seed=11, weight_std=0.05)
+    gm = G.P.Model(**TINY, q_type=q_type, seed=11, weight_std=0.05)
+    assert gm.ffn == om.ffn == 768
+    for sid, kind in streams(TINY["n_layers"]):
+        rows, cols = shape_of(TINY, om.ffn, kind)
+        ow, os_ = om.tensor(sid, rows, cols)
+        gw, gs = gm.tensor(sid, rows, cols)
+        if q_type == 1:
+            assert (ow == gw).all(), sid
+            assert (os_.view(np.uint16) == gs.view(np.uint16)).all(), sid
+        else:
+            assert (ow.view(np.uint16) == gw.view(np.uint16)).all(), sid
+
+
+@pytest.mark.parametrize("cfg", [TINY, SMALL], ids=["tiny", "small"])
+@pytest.mark.parametrize("q_type", [0, 1])
+def test_prefill_and_decode_vs_oracle(gpu, cfg, q_type):
+    G = gpu
+    om = O.Model(**cfg, q_type=q_type, seed=3, weight_std=0.05)
+    gm = G.P.Model(**cfg, q_type=q_type, seed=3, weight_std=0.05)
+    oc = O.Context(om, context_len=64, temperature=0.8)
+    gc = G.P.Context(gm, context_len=64, temperature=0.8)
+    toks = np.random.default_rng(5).integers(0, cfg["n_vocab"], 19).astype(np.int16)
+    feed = toks
+    for step in range(12):
+        otok, ohid, ologits, oprobs = oc.next_token(feed, want=True)
+        gtok = gc.next_token(feed)
+        n = len(feed)
+        assert G.max_abs_rel(gc.hidden(n), ohid) <= TOL, step
+        assert G.max_abs_rel(gc.logits(), ologits) <= TOL, step
+        assert G.max_abs_rel(gc.probs(), oprobs) <= 2 * TOL, step
+        # the device argmax is the first maximum of the device's own fp16 probabilities
+        assert gtok == O.argmax_first(gc.probs())
+        lo = np.sort(ologits.astype(np.float32))
+        if lo[-1] - lo[-2] > 0.05:  # well-separated top-1: must agree
+            assert gtok == otok, step
+        feed = np.array([otok], dtype=np.int16)  # teacher forcing keeps both sides on one sequence
+    T = 19 + 11
+    for layer in (0, cfg["n_layers"] - 1):
+        ok, ov = oc.kv(layer, T)
+        gk, gv = gc.kv(layer, T)
+        assert G.max_abs_rel(gk, ok) <= TOL and G.max_abs_rel(gv, ov) <= TOL
+    assert gc.tokens_left() == 64 - T
+
+
+def test_prefill_chunks_and_decode_agree(gpu):
+    # KV-cache consistency on the device: one 24-token prefill == 10 + 9 prefill then 5 decode steps
+    G = gpu
+    gm = G.P.Model(**SMALL, seed=9, weight_std=0.05)
+    toks = np.random.default_rng(1).integers(0, SMALL["n_vocab"], 24).astype(np.int16)
+    a = G.P.Context(gm, context_len=32, temperature=0.8)
+    a.next_token(toks)
+    la, ha = a.logits(), a.hidden(24)[-1]
+    b = G.P.Context(gm, context_len=32, temperature=0.8)
+    b.next_token(toks[:10])
+    b.next_token(toks[10:19])
+    for t in toks[19:]:
+        b.next_token([t])
+    assert G.max_abs_rel(b.logits(), la) <= TOL
+    assert G.max_abs_rel(b.hidden(1)[0], ha) <= TOL
+    ka, va = a.kv(3, 24)
+    kb, vb = b.kv(3, 24)
+    assert G.max_abs_rel(kb, ka) <= TOL and G.max_abs_rel(vb, va) <= TOL
+
+
+def test_context_api_behaviour(gpu):
+    G = gpu
+    gm = G.P.Model(**TINY, seed=1)
+    c = G.P.Context(gm, context_len=8, temperature=0.8)
+    assert c.tokens_left() == 8
+    t1 = c.next_token([1, 2, 3])
+    assert c.tokens_left() == 5
+    assert c.next_token(list(range(6))) == -1  # does not fit: the reference asserts
+    assert c.next_token([400]) == -1           # id outside the vocabulary
+    assert c.tokens_left() == 5
+    c.clear_tokens()
+    assert c.tokens_left() == 8 and c.next_token([1, 2, 3]) == t1
+    assert c.memory_usage() > 2 * 2 * 8 * 256 * 2
+
+
+def test_one_llama7b_layer_prefill_512_then_decode_at_2048(gpu):
+    """One LLaMA-7B decoder layer: 512-token prefill, chunked prefill up to 2047 cached tokens,
+    then a single-token decode at KV length 2048."""
+    G = gpu
+    cfg = dict(dim=4096, multiple_of=256, n_heads=32, n_layers=1, n_vocab=1024)
+    om = O.Model(**cfg, seed=0, weight_std=0.02)
+    gm = G.P.Model(**cfg, seed=0, weight_std=0.02)
+    assert gm.ffn == 11008
+    oc = O.Context(om, context_len=2048, temperature=0.8)
+    gc = G.P.Context(gm, context_len=2048, temperature=0.8)
+    toks = np.random.default_rng(0).integers(0, cfg["n_vocab"], 2048).astype(np.int16)
+    otok, ohid, ologits, oprobs = oc.next_token(toks[:512], want=True)
+    gc.next_token(toks[:512])
+    assert G.max_abs_rel(gc.hidden(512), ohid) <= TOL
+    assert G.max_abs_rel(gc.logits(), ologits) <= TOL
+    for a, b in ((512, 1024), (1024, 1536), (1536, 2047)):
+        oc.next_token(toks[a:b])
+        gc.next_token(toks[a:b])
+    otok, ohid, ologits, oprobs = oc.next_token(toks[2047:], want=True)
+    gc.next_token(toks[2047:])
+    assert gc.tokens_left() == 0
+    assert G.max_abs_rel(gc.hidden(1), ohid) <= TOL
+    assert G.max_abs_rel(gc.logits(), ologits) <= TOL
+    ok, ov = oc.kv(0, 2048)
+    gk, gv = gc.kv(0, 2048)
+    assert G.max_abs_rel(gk, ok) <= TOL and G.max_abs_rel(gv, ov) <= TOL
+
+
+def greedy_case(G, name):
+    path = os.path.join(GOLDEN, name)
+    if not os.path.exists(path):
+        pytest.skip("fixture %s not generated" % name)
+    fx = json.load(open(path))
+    gm = G.P.Model(dim=fx["dim"], multiple_of=fx["multiple_of"], n_heads=fx["n_heads"], n_layers=fx["n_layers"],
+                   n_vocab=fx["n_vocab"], norm_eps=fx["norm_eps"], q_type=fx["q_type"], qblock=fx["qblock"],
+                   seed=fx["seed"], weight_std=fx["weight_std"])
+    gc = G.P.Context(gm, context_len=fx["context_len"], temperature=fx["temperature"])
+    feed = np.array(fx["prompt"], dtype=np.int16)
+    got, report = [], []
+    for step, want in enumerate(fx["tokens"]):
+        tok = gc.next_token(feed)
+        got.append(tok)
+        if tok != want:
+            l1, l2, p1, p2 = fx["top2_logits_probs"][step]
+            report.append("step %d: device %d, oracle %d; oracle top-2 logits %.5f / %.5f (margin %.5f)"
+                          % (step, tok, want, l1, l2, l1 - l2))
+        feed = np.array([want], dtype=np.int16)  # teacher forcing: every step is compared on the oracle's sequence
+    gc.close()
+    gm.close()
+    return got, fx["tokens"], report
+
+
+def test_greedy_tokens_llama7b_fp16(gpu):
+    """Full LLaMA-7B shape, fp16: 512-token prompt, 128 greedy steps identical to the oracle's."""
+    got, want, report = greedy_case(gpu, "llama7b_fp16_seed0_greedy.json")
+    assert got == want, "\n".join(report)
+
+
+def test_greedy_tokens_llama30b_u8(gpu):
+    """LLaMA-30B shape, uint8 weights: 512-token prompt, 128 greedy steps identical to the oracle's."""
+    got, want, report = greedy_case(gpu, "llama30b_u8_seed0_greedy.json")
+    assert got == want, "\n".join(report)

@@ -1,0 +1,357 @@
+"""GPU parity of every kernel behind the C ABI against the CPU oracle, on the same seeded inputs.
+
+Bars: bit-exact for the quantiser's codes and scales, for dequantisation, embedding, RoPE and the
+argmax; max-abs-rel <= 1e-2 for every fp16 output that accumulates in fp32 (matmul, attention,
+softmax, norm, silu)."""
+import numpy as np
+import pytest
+
+import oracle_lib as O
+
+pytestmark = pytest.mark.gpu
+
+TOL = 1e-2  # max-abs-rel bar for fp16 outputs with fp32 accumulation
+
+
+@pytest.fixture(scope="module", autouse=True)
+def gpu():
+    import gpu_helpers as G
+    G.setup()
+    yield G
+    G.release()
+
+
+def normal(shape, seed, stream, std):
+    n = int(np.prod(shape))
+    return O.fill_normal_f16(n, seed, stream, std).reshape(shape)
+
+
+def test_fill_normal_matches_oracle_bits(gpu):
+    G = gpu
+    for n, seed, stream, std in [(1000, 0, 1, 0.02), (1 << 20, 7, 33, 1.0), (12345, 2 ** 40 + 3, 2 ** 33, 0.5)]:
+        buf = G.empty((n,))
+        G.B.check(G.L().lcu_fill_normal_f16(buf.ptr, n, seed, stream, std, None))
+        got = G.host(buf, (n,))
+        assert (got.view(np.uint16) == O.fill_normal_f16(n, seed, stream, std).view(np.uint16)).all()
+
+
+@pytest.mark.parametrize("rows,cols,block", [(64, 1024, 128), (7, 512, 32), (5, 2048, 1024), (33, 768, 256)])
+def test_quantize_bit_exact(gpu, rows, cols, block):
+    G = gpu
+    w = normal((rows, cols), 3, 5, 0.02)
+    w[0, :block] = 0  # an all-zero block
+    w[1, 3] = np.float16(65504.0)
+    w[2, :block] = np.float16(6e-8)  # scale underflows to zero
+    codes_d, scales_d = G.empty((rows, cols), np.uint8), G.empty((rows, cols // block))
+    wd = G.dev(w)
+    G.B.check(G.L().lcu_quantize_absmax_u8(codes_d.ptr, scales_d.ptr, wd.ptr, rows, cols, block, None))
+    codes, scales = G.host(codes_d, (rows, cols), np.uint8), G.host(scales_d, (rows, cols // block))
+    ec, es = O.quantize_absmax_u8(w, block)
+    assert (scales.view(np.uint16) == es.view(np.uint16)).all()
+    assert (codes == ec).all()
+    out_d = G.empty((rows, cols))
+    G.B.check(G.L().lcu_dequantize_absmax_u8(out_d.ptr, scales_d.ptr, codes_d.ptr, rows, cols, block, None))
+    assert (G.host(out_d, (rows, cols)).view(np.uint16) == O.dequantize_absmax_u8(ec, es, block).view(np.uint16)).all()
+
+
+def test_quantize_exhaustive_inputs_bit_exact(gpu):
+    G = gpu
+    allbits = np.arange(65536, dtype=np.uint16).view(np.float16)
+    finite = allbits[np.isfinite(allbits)]
+    for absmax in [np.float16(65504.0), np.float16(1.0), np.float16(0.0604), np.float16(3e-4)]:
+        xs = finite[np.abs(finite) <= absmax]
+        n = (len(xs) + 126) // 127
+        blocks = np.zeros((n, 128), dtype=np.float16)
+        blocks[:, 0] = absmax
+        flat = np.zeros(n * 127, dtype=np.float16)
+        flat[: len(xs)] = xs
+        blocks[:, 1:] = flat.reshape(n, 127)
+        codes_d, scales_d = G.empty((n, 128), np.uint8), G.empty((n, 1))
+        G.B.check(G.L().lcu_quantize_absmax_u8(codes_d.ptr, scales_d.ptr, G.dev_keep(blocks).ptr, n, 128, 128, None))
+        ec, es = O.quantize_absmax_u8(blocks, 128)
+        assert (G.host(codes_d, (n, 128), np.uint8) == ec).all()
+        assert (G.host(scales_d, (n, 1)).view(np.uint16) == es.view(np.uint16)).all()
+
+
+def test_dequantize_all_codes_all_scales_bit_exact(gpu):
+    G = gpu
+    # every code against a sweep of scales including subnormal ones
+    scales = np.concatenate([np.arange(0, 0x0500, 7, dtype=np.uint16), np.arange(0x0500, 0x5C00, 97, dtype=np.uint16)])
+    scales = scales.view(np.float16).reshape(-1, 1)
+    n = len(scales)
+    codes = np.tile(np.arange(256, dtype=np.uint8), (n, 1))
+    out_d = G.empty((n, 256))
+    G.B.check(G.L().lcu_dequantize_absmax_u8(out_d.ptr, G.dev_keep(scales).ptr, G.dev_keep(codes).ptr, n, 256, 256, None))
+    assert (G.host(out_d, (n, 256)).view(np.uint16) == O.dequantize_absmax_u8(codes, scales, 256).view(np.uint16)).all()
+
+
+GEMV_SHAPES = [(4096, 11008), (4096, 4096), (11008, 4096), (256, 40), (1032, 77), (6656, 6656)]
+
+
+@pytest.mark.parametrize("K,N", GEMV_SHAPES)
+def test_gemv_f16(gpu, K, N):
+    G = gpu
+    x = normal((1, K), 0, 100, 1.0)
+    w = normal((N, K), 0, 101, 0.02)
+    got = G.gemm_f16(x, w)
+    ref = O.matmul_nt(x, w)
+    assert G.max_abs_rel(got, ref) <= TOL
+    assert G.ulp_mismatch(got, ref) < 0.05  # same fp16 value except where fp32 summation order flips a rounding
+    old = normal((1, N), 0, 102, 1.0)
+    got = G.gemm_f16(x, w, beta=1.0, out=old)
+    assert G.max_abs_rel(got, O.matmul_nt(x, w, beta=1.0, out=old)) <= TOL
+    G.release()
+
+
+def test_gemv_exact_cases(gpu):
+    G = gpu
+    K = 512
+    x = normal((1, K), 1, 1, 1.0)
+    assert (G.gemm_f16(x, np.eye(K, dtype=np.float16)).view(np.uint16) == x.view(np.uint16)).all()
+    w = normal((300, K), 1, 2, 0.02)
+    onehot = np.zeros((1, K), dtype=np.float16)
+    onehot[0, 129] = 1
+    assert (G.gemm_f16(onehot, w)[0].view(np.uint16) == w[:, 129].view(np.uint16)).all()
+    G.release()
+
+
+@pytest.mark.parametrize("K,N", [(4096, 4096), (4096, 11008), (11008, 4096), (256, 40), (1024 + 128, 77), (6656, 17920)])
+def test_gemv_u8(gpu, K, N):
+    G = gpu
+    x = normal((1, K), 0, 200, 1.0)
+    w = normal((N, K), 0, 201, 0.02)
+    codes, scales = O.quantize_absmax_u8(w, 128)
+    got = G.gemm_u8(x, codes, scales, 128)
+    ref = O.matmul_nt_u8(x, codes, scales, 128)
+    assert G.max_abs_rel(got, ref) <= TOL
+    assert G.ulp_mismatch(got, ref) < 0.05
+    old = normal((1, N), 0, 202, 1.0)
+    got = G.gemm_u8(x, codes, scales, 128, beta=1.0, out=old)
+    assert G.max_abs_rel(got, O.matmul_nt_u8(x, codes, scales, 128, beta=1.0, out=old)) <= TOL
+    G.release()
+
+
+def test_gemv_u8_dequant_is_exact(gpu):
+    # one-hot x picks single dequantised weights: they must be the reference's fp16 values exactly
+    G = gpu
+    K, N = 256, 64
+    w = normal((N, K), 4, 1, 0.02)
+    w[:, 128:] *= np.float16(1e-3)  # small scales, some products subnormal in fp16
+    codes, scales = O.quantize_absmax_u8(w, 128)
+    deq = O.dequantize_absmax_u8(codes, scales, 128)
+    for k in (0, 5, 127, 128, 200, 255):
+        x = np.zeros((1, K), dtype=np.float16)
+        x[0, k] = 1
+        got = G.gemm_u8(x, codes, scales, 128)[0]
+        assert (got.view(np.uint16) == deq[:, k].view(np.uint16)).all(), k
+    G.release()
+
+
+@pytest.mark.parametrize("M,K,N", [(512, 4096, 4096), (512, 4096, 11008), (512, 11008, 4096), (128, 256, 128),
+                                   (7, 64, 24), (130, 200, 70), (33, 1024, 257)])
+def test_gemm_f16(gpu, M, K, N):
+    G = gpu
+    x = normal((M, K), 0, 300, 1.0)
+    w = normal((N, K), 0, 301, 0.02)
+    got = G.gemm_f16(x, w)
+    ref = O.matmul_nt(x, w)
+    assert G.max_abs_rel(got, ref) <= TOL
+    assert G.ulp_mismatch(got, ref) < 0.05
+    old = normal((M, N), 0, 302, 1.0)
+    got = G.gemm_f16(x, w, beta=1.0, out=old)
+    assert G.max_abs_rel(got, O.matmul_nt(x, w, beta=1.0, out=old)) <= TOL
+    G.release()
+
+
+def test_gemm_exact_cases(gpu):
+    G = gpu
+    K = 256
+    x = normal((40, K), 2, 1, 1.0)
+    assert (G.gemm_f16(x, np.eye(K, dtype=np.float16)).view(np.uint16) == x.view(np.uint16)).all()
+    # asymmetric operands: out[m, n] pairs lhs row m with rhs row n
+    w = np.zeros((96, K), dtype=np.float16)
+    w[70, 5] = 2
+    x2 = np.zeros((40, K), dtype=np.float16)
+    x2[33, 5] = 3
+    out = G.gemm_f16(x2, w)
+    assert out[33, 70] == 6 and np.count_nonzero(out) == 1
+    G.release()
+
+
+@pytest.mark.parametrize("M,K,N", [(512, 4096, 4096), (512, 4096, 11008), (512, 11008, 4096), (16, 256, 128),
+                                   (130, 384, 70)])
+def test_gemm_u8(gpu, M, K, N):
+    G = gpu
+    x = normal((M, K), 0, 400, 1.0)
+    w = normal((N, K), 0, 401, 0.02)
+    codes, scales = O.quantize_absmax_u8(w, 128)
+    got = G.gemm_u8(x, codes, scales, 128)
+    ref = O.matmul_nt_u8(x, codes, scales, 128)
+    assert G.max_abs_rel(got, ref) <= TOL
+    assert G.ulp_mismatch(got, ref) < 0.05
+    # row r of the M-row product equals the single-row product (decode path) within tolerance
+    one = G.gemm_u8(x[3:4], codes, scales, 128)
+    assert G.max_abs_rel(one, got[3:4]) <= TOL
+    G.release()
+
+
+def test_gemm_rejects_bad_shapes(gpu):
+    G = gpu
+    a = G.dev(np.zeros((4, 12), dtype=np.float16))
+    assert G.L().lcu_gemm_f16_nt(a.ptr, a.ptr, a.ptr, 4, 12, 4, 0.0, None) == -2  # K % 8
+    assert G.L().lcu_gemm_f16_nt(None, a.ptr, a.ptr, 4, 16, 4, 0.0, None) == -2
+    assert G.L().lcu_gemm_f16u8_nt(a.ptr, a.ptr, a.ptr, a.ptr, 1, 256, 4, 100, 0.0, None) == -2
+    assert b"lcu_gemm_f16u8_nt" in G.L().lcu_last_error()
+    assert G.L().lcu_gemm_f16_nt(a.ptr, a.ptr, a.ptr, 0, 16, 4, 0.0, None) == 0  # empty input is fine
+
+
+@pytest.mark.parametrize("rows,cols", [(1, 4096), (512, 4096), (3, 6656), (5, 200)])
+def test_rmsnorm(gpu, rows, cols):
+    G = gpu
+    x = normal((rows, cols), 0, 500, 1.0)
+    w = (normal((cols,), 0, 501, 0.1).astype(np.float32) + 1).astype(np.float16)
+    out_d = G.empty((rows, cols))
+    G.B.check(G.L().lcu_rmsnorm(out_d.ptr, G.dev_keep(x).ptr, G.dev_keep(w).ptr, rows, cols, 1e-6, None))
+    got = G.host(out_d, (rows, cols))
+    ref = O.rms_norm(x, w, 1e-6)
+    assert G.max_abs_rel(got, ref) <= TOL
+    # same reduction order and IEEE 1/sqrt on both sides
+    assert G.ulp_mismatch(got, ref) == 0.0
+    G.release()
+
+
+@pytest.mark.parametrize("rows,pos", [(1, 0), (1, 1337), (512, 0), (40, 2000)])
+def test_rope_bit_exact(gpu, rows, pos):
+    G = gpu
+    heads, dim = 32, 4096
+    x = normal((rows, dim), 0, 600, 1.0)
+    tab = G.B.vp()
+    G.B.check(G.L().lcu_rope_table_create(G.B.C.byref(tab), 2048, 128, 10000.0))
+    out_d = G.empty((rows, dim))
+    G.B.check(G.L().lcu_rope(out_d.ptr, G.dev_keep(x).ptr, rows, dim, heads, pos, tab, 2048, None))
+    got = G.host(out_d, (rows, dim))
+    assert G.ulp_mismatch(got, O.rotary(x, heads, pos_offset=pos)) == 0.0
+    # in place
+    xd = G.dev(x)
+    G.B.check(G.L().lcu_rope(xd.ptr, xd.ptr, rows, dim, heads, pos, tab, 2048, None))
+    assert G.ulp_mismatch(G.host(xd, (rows, dim)), got) == 0.0
+    assert G.L().lcu_rope(xd.ptr, xd.ptr, rows, dim, heads, 2048 - rows + 1, tab, 2048, None) == -2  # past the table
+    G.release()
+    G.L().lcu_free(tab)
+
+
+@pytest.mark.parametrize("rows,w,temp", [(1, 32000, 0.8), (64, 512, 1.0), (3, 77, 1.0), (2, 2048, 0.9)])
+def test_softmax_rows(gpu, rows, w, temp):
+    G = gpu
+    x = normal((rows, w), 0, 700, 2.0)
+    if w > 100:
+        x[:, w - 30:] = -np.inf
+    out_d = G.empty((rows, w))
+    G.B.check(G.L().lcu_softmax_rows(out_d.ptr, G.dev_keep(x).ptr, rows, w, temp, None))
+    got = G.host(out_d, (rows, w))
+    ref = O.softmax_rows(x, temp)
+    assert G.max_abs_rel(got, ref) <= TOL
+    assert G.ulp_mismatch(got, ref) < 0.02
+    if w > 100:
+        assert (got[:, w - 30:] == 0).all()
+    G.release()
+
+
+def test_silu_mul(gpu):
+    G = gpu
+    n = 512 * 11008
+    a, b = normal((n,), 0, 800, 2.0), normal((n,), 0, 801, 1.0)
+    out_d = G.empty((n,))
+    G.B.check(G.L().lcu_silu_mul(out_d.ptr, G.dev_keep(a).ptr, G.dev_keep(b).ptr, n, None))
+    got = G.host(out_d, (n,))
+    ref = O.silu_mul(a, b)
+    assert G.max_abs_rel(got, ref) <= TOL
+    assert G.ulp_mismatch(got, ref) < 0.01
+    G.release()
+
+
+def test_embed_bit_exact(gpu):
+    G = gpu
+    vocab, dim = 1000, 512
+    table = normal((vocab, dim), 0, 900, 0.02)
+    ids = np.array([0, 999, 5, 5, 123], dtype=np.int16)
+    out_d = G.empty((len(ids), dim))
+    G.B.check(G.L().lcu_embed(out_d.ptr, G.dev_keep(ids).ptr, len(ids), dim, G.dev_keep(table).ptr, vocab, None))
+    assert G.ulp_mismatch(G.host(out_d, (len(ids), dim)), O.embed(ids, table)) == 0.0
+    codes, scales = O.quantize_absmax_u8(table, 128)
+    G.B.check(G.L().lcu_embed_u8(out_d.ptr, G.dev_keep(ids).ptr, len(ids), dim, G.dev_keep(codes).ptr,
+                                 G.dev_keep(scales).ptr, 128, vocab, None))
+    assert G.ulp_mismatch(G.host(out_d, (len(ids), dim)), O.embed_u8(ids, codes, scales, 128)) == 0.0
+    # an id outside the table gives zeros, not a stray read
+    bad = np.array([1000, -1], dtype=np.int16)
+    G.B.check(G.L().lcu_embed(out_d.ptr, G.dev_keep(bad).ptr, 2, dim, G.dev_keep(table).ptr, vocab, None))
+    assert (G.host(out_d, (2, dim)) == 0).all()
+    G.release()
+
+
+def test_argmax_first_maximum(gpu):
+    G = gpu
+    out_d = G.empty((1,), np.int32)
+    rng = np.random.default_rng(0)
+    for n in (5, 1024, 32000, 40001):
+        p = rng.random(n).astype(np.float16)
+        m = p.max()
+        ties = rng.choice(n, size=min(4, n), replace=False)
+        p[ties] = m
+        G.B.check(G.L().lcu_argmax_f16(out_d.ptr, G.dev_keep(p).ptr, n, None))
+        expected = int(np.flatnonzero(p == m)[0])
+        assert int(G.host(out_d, (1,), np.int32)[0]) == O.argmax_first(p) == expected
+    G.release()
+
+
+def test_memset_and_copies(gpu):
+    G = gpu
+    for n in (1, 15, 16, 17, 4099, 1 << 20):
+        buf = G.empty((n + 32,), np.uint8)
+        G.B.check(G.L().lcu_memset(buf.ptr, 0xAB, n + 32, None))
+        G.B.check(G.L().lcu_memset(buf.ptr + 3, 0x11, n, None))
+        h = G.host(buf, (n + 32,), np.uint8)
+        assert (h[:3] == 0xAB).all() and (h[3:3 + n] == 0x11).all() and (h[3 + n:] == 0xAB).all()
+
+
+ATT_CASES = [(1, 1), (1, 2), (1, 255), (1, 256), (1, 257), (1, 577), (1, 2048), (5, 5), (64, 64), (70, 70),
+             (512, 512), (3, 130), (40, 300)]
+
+
+@pytest.mark.parametrize("n,T", ATT_CASES)
+def test_attention(gpu, n, T):
+    G = gpu
+    heads, dim = 4, 512
+    start = T - n
+    q = normal((n, dim), 0, 1000, 1.0)
+    k = normal((T, dim), 0, 1001, 1.0)
+    v = normal((T, dim), 0, 1002, 1.0)
+    out_d = G.empty((n, dim))
+    G.B.check(G.L().lcu_attention(out_d.ptr, G.dev_keep(q).ptr, G.dev_keep(k).ptr, G.dev_keep(v).ptr, n, T, start, dim,
+                                  heads, None))
+    got = G.host(out_d, (n, dim))
+    ref = O.attention(q, k, v, heads, start)
+    assert G.max_abs_rel(got, ref) <= TOL
+    if start == 0:
+        assert G.ulp_mismatch(got[0], v[0]) == 0.0  # causal row 0 sees only itself
+    G.release()
+
+
+def test_attention_decode_twice_reuses_workspace(gpu):
+    # the split-T decode path keeps arrival counters in a workspace; back-to-back calls must agree
+    G = gpu
+    heads, dim, T = 32, 4096, 2048
+    q = normal((1, dim), 0, 1100, 1.0)
+    k = normal((T, dim), 0, 1101, 1.0)
+    v = normal((T, dim), 0, 1102, 1.0)
+    kd, vd, qd = G.dev_keep(k), G.dev_keep(v), G.dev_keep(q)
+    ref = O.attention(q, k, v, heads, T - 1)
+    out_d = G.empty((1, dim))
+    for T_use in (T, 700, T):
+        G.B.check(G.L().lcu_attention(out_d.ptr, qd.ptr, kd.ptr, vd.ptr, 1, T_use, T_use - 1, dim, heads, None))
+        got = G.host(out_d, (1, dim))
+        want = ref if T_use == T else O.attention(q, k[:T_use], v[:T_use], heads, T_use - 1)
+        assert G.max_abs_rel(got, want) <= TOL
+    assert G.L().lcu_attention(out_d.ptr, qd.ptr, kd.ptr, vd.ptr, 1, 10, 5, dim, heads, None) == -2
+    assert G.L().lcu_attention(out_d.ptr, qd.ptr, kd.ptr, vd.ptr, 1, 10, 9, dim, 31, None) == -2
+    G.release()

@@ -33,6 +33,12 @@ uint32_t lcu_model_ffn_dim(const lcu_model*);                      /* llama_para
  * wq wk wv wo w1 w2 w3; `scales` may be NULL for fp16 models */
 int lcu_model_read_tensor(const lcu_model*, uint64_t stream_id, void* values, void* scales);
 
+/* device pointers of a weight matrix (values or codes, and scales or NULL) and of the norm weight
+ * vectors: which = -1 final norm, 2l attention_norm of layer l, 2l+1 ffn_norm of layer l.  Borrowed;
+ * valid while the model lives.  For benchmarks that launch single kernels on the real weights. */
+int lcu_model_tensor_ptr(const lcu_model*, uint64_t stream_id, void** values_dev, void** scales_dev);
+void* lcu_model_norm_ptr(const lcu_model*, int which);
+
 lcu_context* lcu_context_create(lcu_model*, int context_len, float temperature);   /* llama_context::create */
 void lcu_context_destroy(lcu_context*);
 void lcu_context_clear_tokens(lcu_context*);                                        /* clear_tokens */

@@ -58,6 +58,13 @@ int lcu_d2d(void* dst_dev, const void* src_dev, size_t bytes, void* stream);
 int lcu_stream_create(void** out_stream);
 int lcu_stream_destroy(void* stream);
 int lcu_sync(void* stream);                                                     /* NULL = whole device */
+/* HIP graph capture of the launches made on `stream` between begin and end; every lcu_* kernel
+ * entry point may be captured (none of them records a memset node or allocates).  No counterpart
+ * in the reference, whose host loop launches ~480 kernels per token one by one. */
+int lcu_graph_begin_capture(void* stream);
+int lcu_graph_end_capture(void* stream, void** out_graph_exec);
+int lcu_graph_launch(void* graph_exec, void* stream);
+int lcu_graph_destroy(void* graph_exec);
 int lcu_event_create(void** out_event);
 int lcu_event_destroy(void* event);
 int lcu_event_record(void* event, void* stream);
@@ -105,6 +112,10 @@ int lcu_embed_u8(void* out_dev, const void* ids_dev, int n_ids, int dim, const v
 /* the host argmax of llama_cu.cu:1205-1209 done on the device: index of the first maximum of n
  * fp16 values compared as float, written as int32 */
 int lcu_argmax_f16(void* out_index_dev, const void* values_dev, int n, void* stream);
+/* softmax_rows over one row of n logits with temperature (launch site 1196) and the argmax of
+ * 1205-1209 on its rounded output, in one launch; probs_dev must not alias logits_dev */
+int lcu_softmax_argmax(void* probs_dev, void* out_index_dev, const void* logits_dev, int n, float temp,
+                       void* stream);
 
 /* ---- attention: matmul_qk + softmax_rows + matmul_qkv, llama_cu.cu:400-531, launch sites
  * 1161-1171, without the [n_heads, n, T] score tensor in memory.  q [n_new, dim]; k (already
@@ -115,15 +126,23 @@ int lcu_argmax_f16(void* out_index_dev, const void* values_dev, int n, void* str
 int lcu_attention(void* out_dev, const void* q_dev, const void* k_dev, const void* v_dev,
                   int n_new, int T, int start_pos, int dim, int n_heads, void* stream);
 
+/* lcu_attention for one new token whose position (= T - 1) is read from the device int32 pos_dev
+ * when the kernel runs; max_T bounds it (the cache length). */
+int lcu_attention_decode(void* out_dev, const void* q_dev, const void* k_dev, const void* v_dev,
+                         const void* pos_dev, int max_T, int dim, int n_heads, void* stream);
+
 /* ---- fused decode steps (n_new == 1), each replacing several launch sites of next_token ---- */
 /* rms_norm(x, attn_norm) -> Wq/Wk/Wv GEMV -> RoPE(q, k at position pos) -> q to q_out, k and v into
  * row pos of the caches: llama_cu.cu:1129-1156.  Weight pointers are fp16 [dim, dim], or uint8 codes
- * with fp16 scales when block > 0. */
+ * with fp16 scales when block > 0.  norm_w_dev == NULL means x_dev is already normalised
+ * (lcu_rmsnorm ran first); the same holds for lcu_decode_ffn_up.  pos_dev != NULL: the position is
+ * read from that device int32 when the kernel runs (`pos` is ignored), so that one captured graph
+ * serves every decode step. */
 int lcu_decode_qkv(void* q_out_dev, void* k_cache_dev, void* v_cache_dev, const void* x_dev,
                    const void* norm_w_dev, const void* wq_dev, const void* wk_dev, const void* wv_dev,
                    const void* sq_dev, const void* sk_dev, const void* sv_dev, int block, int dim,
-                   int n_heads, int pos, float eps, const void* rope_table_dev, int table_positions,
-                   void* stream);
+                   int n_heads, int pos, const void* pos_dev, float eps, const void* rope_table_dev,
+                   int table_positions, void* stream);
 /* rms_norm(x, ffn_norm) -> W1 and W3 GEMV -> silu(w1) * w3: llama_cu.cu:1176-1183 */
 int lcu_decode_ffn_up(void* out_dev, const void* x_dev, const void* norm_w_dev, const void* w1_dev,
                       const void* w3_dev, const void* s1_dev, const void* s3_dev, int block, int dim,

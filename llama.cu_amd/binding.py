@@ -57,8 +57,14 @@ SIGNATURES = {
     "lcu_embed": (i32, [vp, vp, i32, i32, vp, i32, vp]),
     "lcu_embed_u8": (i32, [vp, vp, i32, i32, vp, vp, i32, i32, vp]),
     "lcu_argmax_f16": (i32, [vp, vp, i32, vp]),
+    "lcu_softmax_argmax": (i32, [vp, vp, vp, i32, f32, vp]),
     "lcu_attention": (i32, [vp, vp, vp, vp, i32, i32, i32, i32, i32, vp]),
-    "lcu_decode_qkv": (i32, [vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, i32, i32, i32, i32, f32, vp, i32, vp]),
+    "lcu_decode_qkv": (i32, [vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, i32, i32, i32, i32, vp, f32, vp, i32, vp]),
+    "lcu_attention_decode": (i32, [vp, vp, vp, vp, vp, i32, i32, i32, vp]),
+    "lcu_graph_begin_capture": (i32, [vp]),
+    "lcu_graph_end_capture": (i32, [vp, C.POINTER(vp)]),
+    "lcu_graph_launch": (i32, [vp, vp]),
+    "lcu_graph_destroy": (i32, [vp]),
     "lcu_decode_ffn_up": (i32, [vp, vp, vp, vp, vp, vp, vp, i32, i32, i32, f32, vp]),
     "lcu_decode_logits": (i32, [vp, vp, vp, vp, vp, i32, i32, i32, f32, vp]),
     "lcu_fill_normal_f16": (i32, [vp, sz, u64, u64, f32, vp]),
@@ -69,6 +75,8 @@ SIGNATURES = {
     "lcu_model_destroy": (None, [vp]),
     "lcu_model_ffn_dim": (u32, [vp]),
     "lcu_model_read_tensor": (i32, [vp, u64, vp, vp]),
+    "lcu_model_tensor_ptr": (i32, [vp, u64, C.POINTER(vp), C.POINTER(vp)]),
+    "lcu_model_norm_ptr": (vp, [vp, i32]),
     "lcu_context_create": (vp, [vp, i32, f32]),
     "lcu_context_destroy": (None, [vp]),
     "lcu_context_clear_tokens": (None, [vp]),
@@ -190,6 +198,15 @@ class Model:
         if rc:
             raise LcuError("lcu_model_read_tensor %d" % rc)
         return w, None
+
+    def tensor_ptr(self, stream_id):
+        d, s = vp(), vp()
+        if lib().lcu_model_tensor_ptr(self.h, stream_id, C.byref(d), C.byref(s)):
+            raise LcuError("lcu_model_tensor_ptr")
+        return d.value, s.value
+
+    def norm_ptr(self, which):
+        return lib().lcu_model_norm_ptr(self.h, which)
 
     def close(self):
         if getattr(self, "h", None):

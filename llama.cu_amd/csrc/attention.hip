@@ -9,12 +9,9 @@
 // Layouts: q [n_new, dim]; k, v = first T rows of a [*, dim] cache (K already rotated); head h is
 // columns h*128 .. h*128+127.
 //
-// Decode (n_new == 1), HBM bound, two kernels so that every compute unit streams part of the cache:
-//   scores: grid (T/256, heads); 16 lanes share one cached K row (16 bytes each), fp32 dot,
-//           fp16 score to a workspace
-//   pv:     grid (T/256, heads); every workgroup redoes the cheap row max / exp-sum over all T
-//           scores of its head, forms its 256 probabilities, accumulates p * V for them, and the
-//           last workgroup of a head to arrive adds the partial sums in split order
+// Decode (n_new == 1): one 1024-thread workgroup per head does scores, softmax and the weighted
+// sum in one launch; 16 lanes share one cached row (16 bytes each), 64 rows per pass, 8 passes of
+// loads in flight per thread.
 // Prefill (n_new > 1), matrix-core bound: one workgroup per (32 query rows, head); Q.K^T by
 // v_mfma_f32_16x16x32_f16 into an LDS score strip [32][T], softmax in LDS, P.V by MFMA with V
 // staged transposed in LDS.
@@ -27,105 +24,126 @@ namespace {
 constexpr int HD = 128;            // head_dim
 constexpr int MAX_T_DECODE = 4096;
 constexpr int MAX_HEADS = 64;
-constexpr int SPLIT = 256;         // cache rows per decode workgroup
-constexpr int MAX_SPLITS = MAX_T_DECODE / SPLIT;
+constexpr int DEC_THREADS = 1024;
+constexpr int DEC_GROUPS = DEC_THREADS / 16;  // cache rows per pass: 16 lanes x 16 bytes cover one row of a head
+constexpr int DEC_FLIGHT = 8;                 // passes whose loads are requested together
 
-// workspace carve-up (see lcu_init): scores, partial sums, arrival counters
-constexpr size_t WS_SCORES = 0;
-constexpr size_t WS_PARTIAL = WS_SCORES + (size_t)MAX_HEADS * MAX_T_DECODE * sizeof(half_t);
-constexpr size_t WS_COUNTERS = WS_PARTIAL + (size_t)MAX_HEADS * MAX_SPLITS * HD * sizeof(float);
-constexpr size_t WS_END = WS_COUNTERS + MAX_HEADS * sizeof(int);
-
-__global__ __launch_bounds__(256) void decode_scores_kernel(half_t* __restrict__ scores, const half_t* __restrict__ q,
-                                                            const half_t* __restrict__ k, int T, int dim) {
-  const int h = blockIdx.y;
+// One workgroup per head, the whole attention of one new token in a single launch.  The work is
+// a few hundred KB per head, so the kernel is organised around load latency: 1024 threads, every
+// thread keeps 8 independent 16-byte loads in flight, and the first V rows are requested before
+// the softmax statistics are reduced.
+__global__ __launch_bounds__(DEC_THREADS) void decode_attention_kernel(half_t* __restrict__ out,
+                                                                       const half_t* __restrict__ q,
+                                                                       const half_t* __restrict__ k,
+                                                                       const half_t* __restrict__ v, int T, int dim,
+                                                                       const int* __restrict__ pos_dev) {
+  __shared__ half_t sc[MAX_T_DECODE];
+  if (pos_dev) {  // position kept on the device (graph replay): the new row is row *pos_dev, T is the cap
+    T = min(max(*pos_dev + 1, 1), T);
+  }           // fp16 scores, then fp16 probabilities
+  __shared__ float gsum[DEC_GROUPS][HD + 4];
+  __shared__ float red[16];
+  const int h = blockIdx.x;
   const int tid = threadIdx.x;
-  const int sub = tid & 15, grp = tid >> 4;  // 16 lanes per cache row, 16 rows per pass
+  const int sub = tid & 15, grp = tid >> 4;
+  const half_t* kh = k + h * HD + sub * 8;
+  const half_t* vh = v + h * HD + sub * 8;
   const half8_t qh = *reinterpret_cast<const half8_t*>(q + h * HD + sub * 8);
   float qf[8];
 #pragma unroll
   for (int e = 0; e < 8; ++e) qf[e] = (float)qh[e];
   const float denom = sqrtf((float)HD);
-  const int base = blockIdx.x * SPLIT;
-#pragma unroll 4
-  for (int it = 0; it < SPLIT / 16; ++it) {
-    const int p = base + it * 16 + grp;
-    float s = 0.0f;
-    if (p < T) {
-      const half8_t kv = __builtin_nontemporal_load(reinterpret_cast<const half8_t*>(k + (size_t)p * dim + h * HD + sub * 8));
+
+  // ---- scores, llama_cu.cu:400-428 (no mask: the one new row sees every cached row)
+  for (int p0 = 0; p0 < T; p0 += DEC_GROUPS * DEC_FLIGHT) {
+    half8_t kv[DEC_FLIGHT];
 #pragma unroll
-      for (int e = 0; e < 8; ++e) s = fmaf(qf[e], (float)kv[e], s);
+    for (int f = 0; f < DEC_FLIGHT; ++f) {
+      const int p = p0 + f * DEC_GROUPS + grp;
+      kv[f] = p < T ? __builtin_nontemporal_load(reinterpret_cast<const half8_t*>(kh + (size_t)p * dim))
+                    : (half8_t)(0.0f);
     }
 #pragma unroll
-    for (int off = 8; off > 0; off >>= 1) s += __shfl_xor(s, off, WAVE);
-    if (sub == 0 && p < T) {
-      scores[(size_t)h * MAX_T_DECODE + p] = round_f16(s / denom);  // llama_cu.cu:425
+    for (int f = 0; f < DEC_FLIGHT; ++f) {
+      const int p = p0 + f * DEC_GROUPS + grp;
+      float s = 0.0f;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) s = fmaf(qf[e], (float)kv[f][e], s);
+#pragma unroll
+      for (int off = 8; off > 0; off >>= 1) s += __shfl_xor(s, off, WAVE);
+      if (sub == 0 && p < T) sc[p] = round_f16(s / denom);  // 425
     }
   }
-}
+  // first V rows: independent of the statistics below
+  half8_t vv[DEC_FLIGHT];
+#pragma unroll
+  for (int f = 0; f < DEC_FLIGHT; ++f) {
+    const int p = f * DEC_GROUPS + grp;
+    vv[f] = p < T ? __builtin_nontemporal_load(reinterpret_cast<const half8_t*>(vh + (size_t)p * dim)) : (half8_t)(0.0f);
+  }
+  __syncthreads();
 
-__global__ __launch_bounds__(256) void decode_pv_kernel(half_t* __restrict__ out, const half_t* __restrict__ scores,
-                                                        const half_t* __restrict__ v, float* __restrict__ partial,
-                                                        int* __restrict__ counters, int T, int dim, int nsplit) {
-  __shared__ float red[8];
-  __shared__ float gsum[16][HD];
-  __shared__ int s_last;
-  const int h = blockIdx.y, split = blockIdx.x;
-  const int tid = threadIdx.x;
-  const half_t* srow = scores + (size_t)h * MAX_T_DECODE;
-  // softmax_rows statistics over the whole row (llama_cu.cu:442-493), thread t owning t, t+256, ...
+  // ---- softmax_rows, llama_cu.cu:433-499: the first 256 threads play the reference's 256 threads
+  // (thread t owns elements t, t+256, ...), so the exponential sum is associated identically
   float m = -INFINITY;
-  for (int i = tid; i < T; i += 256) m = fmaxf(m, (float)srow[i]);
-  m = block256_max(m, red);
+  if (tid < 256) {
+    for (int i = tid; i < T; i += 256) m = fmaxf(m, (float)sc[i]);
+  }
+  m = wave_max(m);
+  if ((tid & 63) == 0) red[tid >> 6] = m;
+  __syncthreads();
+  m = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));  // wavefronts 4..15 hold -inf
+  __syncthreads();
   float s = 0.0f;
-  for (int i = tid; i < T; i += 256) s += expf((float)srow[i] - m);
-  const float total = block256_sum_ref_order(s, red);
+  if (tid < 256) {
+    for (int i = tid; i < T; i += 256) s += expf((float)sc[i] - m);
+  }
+#pragma unroll
+  for (int off = 16; off > 0; off >>= 1) s += __shfl_xor(s, off, WAVE);
+  if (tid < 256 && (tid & 31) == 0) red[tid >> 5] = s;
+  __syncthreads();
+  float total = red[tid & 7];
+#pragma unroll
+  for (int off = 4; off > 0; off >>= 1) total += __shfl_xor(total, off, WAVE);
+  __syncthreads();
+  for (int i = tid; i < T; i += DEC_THREADS) sc[i] = round_f16(expf((float)sc[i] - m) / total);  // 497
+  __syncthreads();
 
-  const int sub = tid & 15, grp = tid >> 4;
+  // ---- matmul_qkv, llama_cu.cu:511-531: group g adds rows g, g+64, ... in ascending order
   float acc[8];
 #pragma unroll
   for (int e = 0; e < 8; ++e) acc[e] = 0.0f;
-  const int base = split * SPLIT;
-#pragma unroll 4
-  for (int it = 0; it < SPLIT / 16; ++it) {
-    const int p = base + it * 16 + grp;
-    if (p < T) {
-      const float prob = (float)round_f16(expf((float)srow[p] - m) / total);  // rounded as stored, 497
-      const half8_t vv = __builtin_nontemporal_load(reinterpret_cast<const half8_t*>(v + (size_t)p * dim + h * HD + sub * 8));
+  for (int p0 = 0; p0 < T; p0 += DEC_GROUPS * DEC_FLIGHT) {
+    half8_t nv[DEC_FLIGHT];
+    const int n0 = p0 + DEC_GROUPS * DEC_FLIGHT;
+    if (n0 < T) {
 #pragma unroll
-      for (int e = 0; e < 8; ++e) acc[e] = fmaf(prob, (float)vv[e], acc[e]);
+      for (int f = 0; f < DEC_FLIGHT; ++f) {
+        const int p = n0 + f * DEC_GROUPS + grp;
+        nv[f] = p < T ? __builtin_nontemporal_load(reinterpret_cast<const half8_t*>(vh + (size_t)p * dim))
+                      : (half8_t)(0.0f);
+      }
     }
+#pragma unroll
+    for (int f = 0; f < DEC_FLIGHT; ++f) {
+      const int p = p0 + f * DEC_GROUPS + grp;
+      if (p < T) {
+        const float prob = (float)sc[p];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc[e] = fmaf(prob, (float)vv[f][e], acc[e]);
+      }
+    }
+#pragma unroll
+    for (int f = 0; f < DEC_FLIGHT; ++f) vv[f] = nv[f];
   }
 #pragma unroll
   for (int e = 0; e < 8; ++e) gsum[grp][sub * 8 + e] = acc[e];
   __syncthreads();
-  float mine = 0.0f;
   if (tid < HD) {
-#pragma unroll
-    for (int g = 0; g < 16; ++g) mine += gsum[g][tid];
-  }
-  if (nsplit == 1) {
-    if (tid < HD) out[h * HD + tid] = round_f16(mine);
-    return;
-  }
-  if (tid < HD) partial[((size_t)h * MAX_SPLITS + split) * HD + tid] = mine;
-  __threadfence();  // partial sums visible device-wide before the arrival is counted
-  __syncthreads();
-  if (tid == 0) {
-    const int prev = atomicAdd(&counters[h], 1);
-    s_last = (prev == nsplit - 1);
-    if (s_last) counters[h] = 0;  // ready for the next launch
-  }
-  __syncthreads();
-  if (s_last) {
-    __threadfence();
-    if (tid < HD) {
-      float o = 0.0f;
-      for (int sp = 0; sp < nsplit; ++sp) {
-        o += __builtin_nontemporal_load(&partial[((size_t)h * MAX_SPLITS + sp) * HD + tid]);
-      }
-      out[h * HD + tid] = round_f16(o);  // llama_cu.cu:529
-    }
+    float o = 0.0f;
+#pragma unroll 8
+    for (int g = 0; g < DEC_GROUPS; ++g) o += gsum[g][tid];
+    out[h * HD + tid] = round_f16(o);  // 529
   }
 }
 
@@ -285,17 +303,8 @@ int lcu_attention(void* out_dev, const void* q_dev, const void* k_dev, const voi
   hipStream_t s = as_stream(stream);
   if (n_new == 1) {
     LCU_REQUIRE(T <= MAX_T_DECODE, "lcu_attention: T %d exceeds %d", T, MAX_T_DECODE);
-    static_assert(WS_END <= (4u << 20), "workspace too small");
-    unsigned char* ws = (unsigned char*)st->workspace;
-    half_t* scores = (half_t*)(ws + WS_SCORES);
-    float* partial = (float*)(ws + WS_PARTIAL);
-    int* counters = (int*)(ws + WS_COUNTERS);
-    const int nsplit = (T + SPLIT - 1) / SPLIT;
-    dim3 grid(nsplit, n_heads);
-    decode_scores_kernel<<<grid, 256, 0, s>>>(scores, (const half_t*)q_dev, (const half_t*)k_dev, T, dim);
-    LCU_LAUNCH_CHECK();
-    decode_pv_kernel<<<grid, 256, 0, s>>>((half_t*)out_dev, scores, (const half_t*)v_dev, partial, counters, T, dim,
-                                          nsplit);
+    decode_attention_kernel<<<n_heads, DEC_THREADS, 0, s>>>((half_t*)out_dev, (const half_t*)q_dev,
+                                                            (const half_t*)k_dev, (const half_t*)v_dev, T, dim, nullptr);
     LCU_LAUNCH_CHECK();
     return LCU_OK;
   }
@@ -314,6 +323,20 @@ int lcu_attention(void* out_dev, const void* q_dev, const void* k_dev, const voi
   dim3 grid(n_tiles, n_heads);
   prefill_attention_kernel<<<grid, 256, lds, s>>>((half_t*)out_dev, (const half_t*)q_dev, (const half_t*)k_dev,
                                                   (const half_t*)v_dev, n_new, T, start_pos, dim, n_tiles);
+  LCU_LAUNCH_CHECK();
+  return LCU_OK;
+}
+
+int lcu_attention_decode(void* out_dev, const void* q_dev, const void* k_dev, const void* v_dev, const void* pos_dev,
+                         int max_T, int dim, int n_heads, void* stream) {
+  LCU_REQUIRE(out_dev && q_dev && k_dev && v_dev && pos_dev, "lcu_attention_decode: null pointer");
+  LCU_REQUIRE(n_heads > 0 && n_heads <= MAX_HEADS && dim == n_heads * HD,
+              "lcu_attention_decode: dim %d / heads %d unsupported (head_dim must be 128, at most %d heads)", dim,
+              n_heads, MAX_HEADS);
+  LCU_REQUIRE(max_T > 0 && max_T <= MAX_T_DECODE, "lcu_attention_decode: max_T %d outside 1..%d", max_T, MAX_T_DECODE);
+  decode_attention_kernel<<<n_heads, DEC_THREADS, 0, as_stream(stream)>>>(
+      (half_t*)out_dev, (const half_t*)q_dev, (const half_t*)k_dev, (const half_t*)v_dev, max_T, dim,
+      (const int*)pos_dev);
   LCU_LAUNCH_CHECK();
   return LCU_OK;
 }

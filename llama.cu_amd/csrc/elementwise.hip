@@ -12,21 +12,45 @@ namespace {
 // exactly as the reference's (thread t owns elements t, t+256, ...; see block256_sum_ref_order).
 // Two roundings: fp16(x * rms_inv), then fp16(weight * that).
 // ---------------------------------------------------------------------------------------------
-__global__ __launch_bounds__(256) void rmsnorm_kernel(half_t* __restrict__ out, const half_t* __restrict__ in,
+__global__ __launch_bounds__(256) void rmsnorm_kernel(half_t* out, const half_t* in,
                                                       const half_t* __restrict__ weights, int cols, float eps) {
+  extern __shared__ half_t xs[];  // the row, so that it is read from memory once, with 16-byte loads
   __shared__ float red[8];
   const half_t* x = in + (size_t)blockIdx.x * cols;
   half_t* y = out + (size_t)blockIdx.x * cols;
+  const bool vec = (cols % 8) == 0;
+  if (vec) {
+    for (int i = threadIdx.x * 8; i < cols; i += 256 * 8) {
+      *reinterpret_cast<uint4*>(xs + i) = *reinterpret_cast<const uint4*>(x + i);
+    }
+  } else {
+    for (int i = threadIdx.x; i < cols; i += 256) xs[i] = x[i];
+  }
+  __syncthreads();
   float s = 0.0f;
   for (int i = threadIdx.x; i < cols; i += 256) {
-    float v = (float)x[i];
+    float v = (float)xs[i];
     s = fmaf(v, v, s);
   }
   const float total = block256_sum_ref_order(s, red);
   const float rms_inv = 1.0f / sqrtf(total / (float)cols + eps);
-  for (int i = threadIdx.x; i < cols; i += 256) {
-    half_t inner = round_f16((float)x[i] * rms_inv);
-    y[i] = round_f16((float)weights[i] * (float)inner);
+  if (vec) {
+    for (int i = threadIdx.x * 8; i < cols; i += 256 * 8) {
+      const half8_t xv = *reinterpret_cast<const half8_t*>(xs + i);
+      const half8_t wv = *reinterpret_cast<const half8_t*>(weights + i);
+      half8_t r;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const half_t inner = round_f16((float)xv[e] * rms_inv);
+        r[e] = round_f16((float)wv[e] * (float)inner);
+      }
+      *reinterpret_cast<half8_t*>(y + i) = r;
+    }
+  } else {
+    for (int i = threadIdx.x; i < cols; i += 256) {
+      half_t inner = round_f16((float)xs[i] * rms_inv);
+      y[i] = round_f16((float)weights[i] * (float)inner);
+    }
   }
 }
 
@@ -70,6 +94,94 @@ __global__ __launch_bounds__(256) void softmax_rows_kernel(half_t* out, const ha
   const float total = block256_sum_ref_order(s, red);
   for (int i = threadIdx.x; i < w; i += 256) {
     y[i] = round_f16(expf((float)x[i] / temp - m) / total);
+  }
+}
+
+// softmax_rows with temperature over one long row (the logits, llama_cu.cu:1196-1197) followed by
+// the first-maximum argmax of the rounded probabilities (1205-1209), in one 1024-thread
+// workgroup with 16-byte loads.  The exponential sum is associated differently from the
+// 256-thread reference kernel (per-thread partials, then wavefronts, then 16 wavefront sums in
+// order), which moves a probability by at most the last fp32 bit of the sum.
+__global__ __launch_bounds__(1024) void softmax_argmax_kernel(half_t* __restrict__ probs, int* __restrict__ index,
+                                                              const half_t* __restrict__ logits, int n, float temp) {
+  __shared__ float sred[16];
+  __shared__ int sidx[16];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int n8 = n / 8;
+  float m = -INFINITY;
+  for (int c = tid; c < n8; c += 1024) {
+    const half8_t v = *reinterpret_cast<const half8_t*>(logits + (size_t)c * 8);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) m = fmaxf(m, (float)v[e] / temp);
+  }
+  for (int i = n8 * 8 + tid; i < n; i += 1024) m = fmaxf(m, (float)logits[i] / temp);
+  m = wave_max(m);
+  if (lane == 0) sred[wave] = m;
+  __syncthreads();
+  m = sred[0];
+#pragma unroll
+  for (int w = 1; w < 16; ++w) m = fmaxf(m, sred[w]);
+  __syncthreads();
+  float s = 0.0f;
+  for (int c = tid; c < n8; c += 1024) {
+    const half8_t v = *reinterpret_cast<const half8_t*>(logits + (size_t)c * 8);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) s += expf((float)v[e] / temp - m);
+  }
+  for (int i = n8 * 8 + tid; i < n; i += 1024) s += expf((float)logits[i] / temp - m);
+  s = wave_sum(s);
+  if (lane == 0) sred[wave] = s;
+  __syncthreads();
+  float total = 0.0f;
+#pragma unroll
+  for (int w = 0; w < 16; ++w) total += sred[w];
+  __syncthreads();
+  float best = -INFINITY;
+  int idx = 0x7fffffff;
+  for (int c = tid; c < n8; c += 1024) {
+    const half8_t v = *reinterpret_cast<const half8_t*>(logits + (size_t)c * 8);
+    half8_t p;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      p[e] = round_f16(expf((float)v[e] / temp - m) / total);
+      const float f = (float)p[e];
+      if (f > best) {  // ascending index within a thread: strict > keeps the first maximum
+        best = f;
+        idx = c * 8 + e;
+      }
+    }
+    *reinterpret_cast<half8_t*>(probs + (size_t)c * 8) = p;
+  }
+  for (int i = n8 * 8 + tid; i < n; i += 1024) {
+    const half_t p = round_f16(expf((float)logits[i] / temp - m) / total);
+    probs[i] = p;
+    if ((float)p > best || ((float)p == best && i < idx)) {
+      best = (float)p;
+      idx = i;
+    }
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) {
+    const float ob = __shfl_xor(best, off, WAVE);
+    const int oi = __shfl_xor(idx, off, WAVE);
+    if (ob > best || (ob == best && oi < idx)) {
+      best = ob;
+      idx = oi;
+    }
+  }
+  if (lane == 0) {
+    sred[wave] = best;
+    sidx[wave] = idx;
+  }
+  __syncthreads();
+  if (tid == 0) {
+    for (int w = 1; w < 16; ++w) {
+      if (sred[w] > best || (sred[w] == best && sidx[w] < idx)) {
+        best = sred[w];
+        idx = sidx[w];
+      }
+    }
+    *index = idx == 0x7fffffff ? 0 : idx;
   }
 }
 
@@ -263,8 +375,9 @@ int lcu_rmsnorm(void* out_dev, const void* in_dev, const void* weights_dev, int 
   LCU_REQUIRE(out_dev && in_dev && weights_dev, "lcu_rmsnorm: null pointer");
   LCU_REQUIRE(rows >= 0 && cols > 0, "lcu_rmsnorm: bad shape %d x %d", rows, cols);
   if (rows == 0) return LCU_OK;
-  rmsnorm_kernel<<<rows, 256, 0, as_stream(stream)>>>((half_t*)out_dev, (const half_t*)in_dev,
-                                                      (const half_t*)weights_dev, cols, eps);
+  LCU_REQUIRE(cols <= 24576, "lcu_rmsnorm: rows longer than 24576 are not supported");
+  rmsnorm_kernel<<<rows, 256, (size_t)cols * 2, as_stream(stream)>>>((half_t*)out_dev, (const half_t*)in_dev,
+                                                                     (const half_t*)weights_dev, cols, eps);
   LCU_LAUNCH_CHECK();
   return LCU_OK;
 }
@@ -316,6 +429,17 @@ int lcu_softmax_rows(void* out_dev, const void* in_dev, int rows, int w, float t
               (double)temp);
   if (rows == 0) return LCU_OK;
   softmax_rows_kernel<<<rows, 256, 0, as_stream(stream)>>>((half_t*)out_dev, (const half_t*)in_dev, w, temp);
+  LCU_LAUNCH_CHECK();
+  return LCU_OK;
+}
+
+int lcu_softmax_argmax(void* probs_dev, void* out_index_dev, const void* logits_dev, int n, float temp,
+                       void* stream) {
+  LCU_REQUIRE(probs_dev && out_index_dev && logits_dev, "lcu_softmax_argmax: null pointer");
+  LCU_REQUIRE(n > 0 && temp > 0.0f, "lcu_softmax_argmax: bad arguments n %d temp %f", n, (double)temp);
+  LCU_REQUIRE(probs_dev != logits_dev, "lcu_softmax_argmax: probabilities may not overwrite the logits");
+  softmax_argmax_kernel<<<1, 1024, 0, as_stream(stream)>>>((half_t*)probs_dev, (int*)out_index_dev,
+                                                          (const half_t*)logits_dev, n, temp);
   LCU_LAUNCH_CHECK();
   return LCU_OK;
 }

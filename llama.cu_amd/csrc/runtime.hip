@@ -156,6 +156,39 @@ int lcu_sync(void* stream) {
   return LCU_OK;
 }
 
+int lcu_graph_begin_capture(void* stream) {
+  LCU_REQUIRE(stream != nullptr, "lcu_graph_begin_capture: capture needs an explicit stream");
+  LCU_HIP(hipStreamBeginCapture(as_stream(stream), hipStreamCaptureModeThreadLocal));
+  return LCU_OK;
+}
+
+int lcu_graph_end_capture(void* stream, void** out_graph_exec) {
+  LCU_REQUIRE(stream && out_graph_exec, "lcu_graph_end_capture: null argument");
+  hipGraph_t graph = nullptr;
+  LCU_HIP(hipStreamEndCapture(as_stream(stream), &graph));
+  hipGraphExec_t exec = nullptr;
+  hipError_t e = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
+  (void)hipGraphDestroy(graph);
+  if (e != hipSuccess) {
+    return set_error(LCU_E_HIP, "lcu_graph_end_capture: hipGraphInstantiate failed: %s", hipGetErrorString(e));
+  }
+  *out_graph_exec = exec;
+  return LCU_OK;
+}
+
+int lcu_graph_launch(void* graph_exec, void* stream) {
+  LCU_REQUIRE(graph_exec != nullptr, "lcu_graph_launch: null graph");
+  LCU_HIP(hipGraphLaunch(reinterpret_cast<hipGraphExec_t>(graph_exec), as_stream(stream)));
+  return LCU_OK;
+}
+
+int lcu_graph_destroy(void* graph_exec) {
+  if (graph_exec) {
+    LCU_HIP(hipGraphExecDestroy(reinterpret_cast<hipGraphExec_t>(graph_exec)));
+  }
+  return LCU_OK;
+}
+
 int lcu_event_create(void** out_event) {
   LCU_REQUIRE(out_event != nullptr, "lcu_event_create: null output");
   hipEvent_t e;

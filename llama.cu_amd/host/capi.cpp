@@ -87,6 +87,30 @@ int lcu_model_read_tensor(const lcu_model* m, uint64_t stream_id, void* values, 
   return 0;
 }
 
+int lcu_model_tensor_ptr(const lcu_model* m, uint64_t stream_id, void** values_dev, void** scales_dev) {
+  weight_tensor const* t = m->impl()->tensor_by_stream(stream_id);
+  if (!t || !values_dev) {
+    return -1;
+  }
+  *values_dev = t->data.data();
+  if (scales_dev) {
+    *scales_dev = t->scales.data();
+  }
+  return 0;
+}
+
+void* lcu_model_norm_ptr(const lcu_model* m, int which) {
+  llama_model_impl* mi = m->impl();
+  if (which == -1) {
+    return mi->norm.data();
+  }
+  if (which < 0 || (size_t)(which / 2) >= mi->layers.size()) {
+    return nullptr;
+  }
+  llama_layer const& L = mi->layers[which / 2];
+  return (which & 1) ? L.ffn_norm.data() : L.attn_norm.data();
+}
+
 lcu_context* lcu_context_create(lcu_model* m, int context_len, float temperature) {
   if (!m || context_len <= 0 || !(temperature > 0.0f)) {
     return nullptr;

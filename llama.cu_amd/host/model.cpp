@@ -8,6 +8,7 @@
 // every call (K is cached rotated; RoPE depends only on value and position, so the bits agree),
 // and its one-launch-per-operation decode loop (a single new token runs the fused kernels).
 #include <assert.h>
+#include <stddef.h>
 #include <string.h>
 
 #include "model_impl.hpp"
@@ -235,6 +236,7 @@ llama_context_impl::llama_context_impl(llama_model* model, int context_len, floa
 
 llama_context_impl::~llama_context_impl() {
   lcu_sync(stream_);
+  lcu_graph_destroy(decode_graph_);
   lcu_free(rope_table_);
   lcu_stream_destroy(stream_);
 }
@@ -244,6 +246,7 @@ void llama_context_impl::clear_tokens() {
   llama_params const& p = model_->params;
   const size_t ctx = (size_t)context_len_, dim = p.dim, ffn = p.ffn_dim();
   LCU_CHECK(lcu_sync(stream_));
+  drop_graph();  // it holds pointers into the caches released below
   kv_.clear();
   kv_.resize(p.n_layers);
   for (auto& kv : kv_) {
@@ -264,6 +267,7 @@ void llama_context_impl::clear_tokens() {
     t_logits_ = gpu_buffer((size_t)p.n_vocab * 2);
     t_probs_ = gpu_buffer((size_t)p.n_vocab * 2);
     t_argmax_ = gpu_buffer(sizeof(int));
+    t_step_ = gpu_buffer(sizeof(step_state));
   }
   LCU_CHECK(lcu_sync(stream_));
   start_pos_ = 0;
@@ -276,7 +280,7 @@ size_t llama_context_impl::context_memory_usage() {
     count += kv.k.size() + kv.v.size();
   }
   for (gpu_buffer const* b : {&t_embed_, &t_norm_, &t_xq_, &t_out_, &t_w1_, &t_w3_, &t_silu_, &t_tokens_, &t_logits_,
-                              &t_probs_, &t_argmax_}) {
+                              &t_probs_, &t_argmax_, &t_step_}) {
     count += b->size();
   }
   return count;
@@ -292,67 +296,121 @@ void llama_context_impl::matmul(void* out, const void* lhs, weight_tensor const&
   }
 }
 
-short llama_context_impl::next_token(std::vector<short> const& new_tokens) {
+// The layer loop for n new rows sitting in t_embed_; positions start_pos_ .. start_pos_ + n - 1.
+// n == 1 takes the fused decode kernels, which read the position from t_step_ on the device.
+void llama_context_impl::enqueue_layers(int n) {
   llama_params const& p = model_->params;
-  const int n = (int)new_tokens.size();
-  assert(n > 0);
-  assert(new_tokens.size() + start_pos_ <= (size_t)context_len_);  // llama_cu.cu:1074
-  const int dim = p.dim, ffn = p.ffn_dim(), heads = p.n_heads, vocab = p.n_vocab;
+  const int dim = p.dim, ffn = p.ffn_dim(), heads = p.n_heads;
   const int sp = start_pos_, T = sp + n;
   const int block = p.q_type == quantization_type::uint8 ? p.quantization_block_size : 0;
   char* x = (char*)t_embed_.data();
-
-  // 1086-1097
-  LCU_CHECK(lcu_h2d(t_tokens_.data(), new_tokens.data(), n * sizeof(short), stream_));
-  if (model_->tok_embeddings.quantised) {
-    LCU_CHECK(lcu_embed_u8(x, t_tokens_.data(), n, dim, model_->tok_embeddings.data.data(),
-                           model_->tok_embeddings.scales.data(), block, vocab, stream_));
-  } else {
-    LCU_CHECK(lcu_embed(x, t_tokens_.data(), n, dim, model_->tok_embeddings.data.data(), vocab, stream_));
-  }
-
   for (size_t l = 0; l < model_->layers.size(); ++l) {
     llama_layer const& L = model_->layers[l];
     char* kc = (char*)kv_[l].k.data();
     char* vc = (char*)kv_[l].v.data();
-    char* k_new = kc + (size_t)sp * dim * 2;
-    char* v_new = vc + (size_t)sp * dim * 2;
     if (n == 1) {
-      // 1129-1156 in one launch
-      LCU_CHECK(lcu_decode_qkv(t_xq_.data(), kc, vc, x, L.attn_norm.data(), L.wq.data.data(), L.wk.data.data(),
+      // 1129, then 1144-1156 in one launch, then 1161-1171 in one launch
+      LCU_CHECK(lcu_rmsnorm(t_norm_.data(), x, L.attn_norm.data(), 1, dim, p.norm_eps, stream_));
+      LCU_CHECK(lcu_decode_qkv(t_xq_.data(), kc, vc, t_norm_.data(), nullptr, L.wq.data.data(), L.wk.data.data(),
                                L.wv.data.data(), L.wq.scales.data(), L.wk.scales.data(), L.wv.scales.data(), block, dim,
-                               heads, sp, p.norm_eps, rope_table_, context_len_, stream_));
+                               heads, 0, t_step_.data(), p.norm_eps, rope_table_, context_len_, stream_));
+      LCU_CHECK(lcu_attention_decode(t_out_.data(), t_xq_.data(), kc, vc, t_step_.data(), context_len_, dim, heads,
+                                     stream_));
     } else {
+      char* k_new = kc + (size_t)sp * dim * 2;
+      char* v_new = vc + (size_t)sp * dim * 2;
       LCU_CHECK(lcu_rmsnorm(t_norm_.data(), x, L.attn_norm.data(), n, dim, p.norm_eps, stream_));            // 1129
       matmul(t_xq_.data(), t_norm_.data(), L.wq, n, 0.0f);                                                   // 1144
       LCU_CHECK(lcu_rope(t_xq_.data(), t_xq_.data(), n, dim, heads, sp, rope_table_, context_len_, stream_));  // 1146
       matmul(k_new, t_norm_.data(), L.wk, n, 0.0f);                                                          // 1150
       LCU_CHECK(lcu_rope(k_new, k_new, n, dim, heads, sp, rope_table_, context_len_, stream_));  // 1152, new rows only
       matmul(v_new, t_norm_.data(), L.wv, n, 0.0f);                                                          // 1156
+      LCU_CHECK(lcu_attention(t_out_.data(), t_xq_.data(), kc, vc, n, T, sp, dim, heads, stream_));          // 1161-1171
     }
-    LCU_CHECK(lcu_attention(t_out_.data(), t_xq_.data(), kc, vc, n, T, sp, dim, heads, stream_));            // 1161-1171
     matmul(x, t_out_.data(), L.wo, n, 1.0f);                                                                 // 1174
+    LCU_CHECK(lcu_rmsnorm(t_norm_.data(), x, L.ffn_norm.data(), n, dim, p.norm_eps, stream_));               // 1176
     if (n == 1) {
-      // 1176-1183 in one launch
-      LCU_CHECK(lcu_decode_ffn_up(t_silu_.data(), x, L.ffn_norm.data(), L.w1.data.data(), L.w3.data.data(),
+      // 1180-1183 in one launch
+      LCU_CHECK(lcu_decode_ffn_up(t_silu_.data(), t_norm_.data(), nullptr, L.w1.data.data(), L.w3.data.data(),
                                   L.w1.scales.data(), L.w3.scales.data(), block, dim, ffn, p.norm_eps, stream_));
     } else {
-      LCU_CHECK(lcu_rmsnorm(t_norm_.data(), x, L.ffn_norm.data(), n, dim, p.norm_eps, stream_));             // 1176
       matmul(t_w1_.data(), t_norm_.data(), L.w1, n, 0.0f);                                                   // 1180
       matmul(t_w3_.data(), t_norm_.data(), L.w3, n, 0.0f);                                                   // 1181
       LCU_CHECK(lcu_silu_mul(t_silu_.data(), t_w1_.data(), t_w3_.data(), (size_t)n * ffn, stream_));         // 1183
     }
     matmul(x, t_silu_.data(), L.w2, n, 1.0f);                                                                // 1185
   }
-  // 1191-1197: the reference normalises every row and uses the last one
+}
+
+// final norm of the last row, logits, softmax with temperature, argmax: llama_cu.cu:1191-1209.
+// The reference normalises every row and uses the last one.
+void llama_context_impl::enqueue_head(int n) {
+  llama_params const& p = model_->params;
+  const int dim = p.dim, vocab = p.n_vocab;
+  const int block = p.q_type == quantization_type::uint8 ? p.quantization_block_size : 0;
+  char* x = (char*)t_embed_.data();
   LCU_CHECK(lcu_decode_logits(t_logits_.data(), x + (size_t)(n - 1) * dim * 2, model_->norm.data(),
                               model_->output.data.data(), model_->output.scales.data(), block, dim, vocab, p.norm_eps,
                               stream_));
-  LCU_CHECK(lcu_softmax_rows(t_probs_.data(), t_logits_.data(), 1, vocab, temperature_, stream_));
-  // 1198-1209: first maximum of the fp16 probabilities, found on the device; 4 bytes come back
-  LCU_CHECK(lcu_argmax_f16(t_argmax_.data(), t_probs_.data(), vocab, stream_));
+  // the first maximum of the fp16 probabilities is found on the device; 4 bytes go back to the host
+  LCU_CHECK(lcu_softmax_argmax(t_probs_.data(), t_argmax_.data(), t_logits_.data(), vocab, temperature_, stream_));
+}
+
+void llama_context_impl::drop_graph() {
+  if (decode_graph_) {
+    LCU_CHECK(lcu_graph_destroy(decode_graph_));
+    decode_graph_ = nullptr;
+  }
+  decode_calls_ = 0;
+}
+
+short llama_context_impl::next_token(std::vector<short> const& new_tokens) {
+  llama_params const& p = model_->params;
+  const int n = (int)new_tokens.size();
+  assert(n > 0);
+  assert(new_tokens.size() + start_pos_ <= (size_t)context_len_);  // llama_cu.cu:1074
+  const int dim = p.dim, vocab = p.n_vocab;
+  const int block = p.q_type == quantization_type::uint8 ? p.quantization_block_size : 0;
+  char* x = (char*)t_embed_.data();
+  const void* ids = t_tokens_.data();
+  if (n == 1) {
+    host_step_.pos = start_pos_;
+    host_step_.token = new_tokens[0];
+    LCU_CHECK(lcu_h2d(t_step_.data(), &host_step_, sizeof(host_step_), stream_));
+    ids = (char*)t_step_.data() + offsetof(step_state, token);
+  } else {
+    LCU_CHECK(lcu_h2d(t_tokens_.data(), new_tokens.data(), n * sizeof(short), stream_));  // 1086
+  }
+  auto enqueue_all = [&]() {
+    // 1087-1097
+    if (model_->tok_embeddings.quantised) {
+      LCU_CHECK(lcu_embed_u8(x, ids, n, dim, model_->tok_embeddings.data.data(), model_->tok_embeddings.scales.data(),
+                             block, vocab, stream_));
+    } else {
+      LCU_CHECK(lcu_embed(x, ids, n, dim, model_->tok_embeddings.data.data(), vocab, stream_));
+    }
+    enqueue_layers(n);
+    enqueue_head(n);
+  };
+  if (n == 1) {
+    // A decode step is ~260 launches of a few microseconds each: the first one runs eagerly (and
+    // loads the kernels), the second is captured into a HIP graph, every later one replays it.
+    ++decode_calls_;
+    if (!decode_graph_ && decode_calls_ >= 2) {
+      LCU_CHECK(lcu_graph_begin_capture(stream_));
+      enqueue_all();
+      LCU_CHECK(lcu_graph_end_capture(stream_, &decode_graph_));
+    }
+    if (decode_graph_) {
+      LCU_CHECK(lcu_graph_launch(decode_graph_, stream_));
+    } else {
+      enqueue_all();
+    }
+  } else {
+    enqueue_all();
+  }
   int token = 0;
-  LCU_CHECK(lcu_d2h(&token, t_argmax_.data(), sizeof(int), stream_));
+  LCU_CHECK(lcu_d2h(&token, t_argmax_.data(), sizeof(int), stream_));  // 1198-1200, blocks
   start_pos_ += n;
   last_n_ = n;
   return (short)token;

@@ -59,9 +59,22 @@ struct llama_context_impl final : public llama_context {
 
  private:
   void matmul(void* out, const void* lhs, weight_tensor const& w, int M, float beta);
+  void enqueue_layers(int n);
+  void enqueue_head(int n);
+  void drop_graph();
   std::vector<kv_cache_layer> kv_;
   gpu_buffer t_embed_, t_norm_, t_xq_, t_out_, t_w1_, t_w3_, t_silu_;
   gpu_buffer t_tokens_, t_logits_, t_probs_, t_argmax_;
+  // decode step state on the device: {int32 position, int16 token}; the decode kernels read the
+  // position from here, so one captured graph replays for every step
+  gpu_buffer t_step_;
+  struct step_state {
+    int32_t pos;
+    int16_t token;
+    int16_t pad;
+  } host_step_{};
+  void* decode_graph_{nullptr};
+  int decode_calls_{0};
   void* stream_{nullptr};
   void* rope_table_{nullptr};
   int last_n_{0};

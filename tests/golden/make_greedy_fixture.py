@@ -5,8 +5,8 @@
 
 Each fixture holds the model shape, the seeds, the 512 prompt token ids, the 128 greedy tokens the
 oracle produces (tensor-core flavour of the matmul, temperature 0.8 as main.cpp:58), and for every
-step the top-1/top-2 values of the fp16 logits and probabilities, so that a mismatch in a GPU run
-can be attributed to a near-tie.  Only the oracle runs here; nothing from the reference is
+step the two largest fp16 logits with their token ids and the two largest probabilities, so that
+a mismatch in a GPU run can be attributed to a near-tie.  Only the oracle runs here; nothing from the reference is
 imported or executed.
 """
 import json
@@ -39,19 +39,22 @@ def main():
     print("model built in %.1fs (ffn %d)" % (time.time() - t0, model.ffn), flush=True)
     ctx = O.Context(model, context_len=2048, temperature=0.8, flavour=1)
     prompt = np.random.default_rng(seed).integers(0, cfg["n_vocab"], prompt_len).astype(np.int16)
-    tokens, top = [], []
+    tokens, top, top_ids = [], [], []
     feed = prompt
     for step in range(steps):
         t1 = time.time()
         tok, _, logits, probs = ctx.next_token(feed, want=True)
-        lo = np.sort(logits.astype(np.float32))[-2:]
+        lf = logits.astype(np.float32)
+        order = np.argsort(-lf, kind="stable")[:2]  # stable: the lower id first among equals
+        lo = lf[order[::-1]]
         po = np.sort(probs.astype(np.float32))[-2:]
         tokens.append(int(tok))
         top.append([float(lo[1]), float(lo[0]), float(po[1]), float(po[0])])
+        top_ids.append([int(order[0]), int(order[1])])
         feed = np.array([tok], dtype=np.int16)
         print("step %d token %d logit margin %.5f (%.1fs)" % (step, tok, lo[1] - lo[0], time.time() - t1), flush=True)
     out = dict(name=name, seed=seed, weight_std=0.02, norm_eps=1e-6, qblock=128, temperature=0.8, context_len=2048,
-               prompt=[int(t) for t in prompt], tokens=tokens, top2_logits_probs=top, **cfg)
+               prompt=[int(t) for t in prompt], tokens=tokens, top2_logits_probs=top, top2_ids=top_ids, **cfg)
     path = os.path.join(HERE, "%s_seed%d_greedy.json" % (name, seed))
     with open(path, "w") as f:
         json.dump(out, f)

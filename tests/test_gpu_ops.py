@@ -355,3 +355,20 @@ def test_attention_decode_twice_reuses_workspace(gpu):
     assert G.L().lcu_attention(out_d.ptr, qd.ptr, kd.ptr, vd.ptr, 1, 10, 5, dim, heads, None) == -2
     assert G.L().lcu_attention(out_d.ptr, qd.ptr, kd.ptr, vd.ptr, 1, 10, 9, dim, 31, None) == -2
     G.release()
+
+
+@pytest.mark.parametrize("n,temp", [(32000, 0.8), (32003, 0.9), (5, 1.0), (1024, 0.5)])
+def test_softmax_argmax_fused(gpu, n, temp):
+    G = gpu
+    x = normal((1, n), 0, 1200, 1.3)
+    x[0, n // 3] = x.max()  # two equal largest logits: the first index must win
+    x[0, n // 3 * 2] = x.max()
+    probs_d, idx_d = G.empty((n,)), G.empty((1,), np.int32)
+    G.B.check(G.L().lcu_softmax_argmax(probs_d.ptr, idx_d.ptr, G.dev_keep(x).ptr, n, temp, None))
+    got = G.host(probs_d, (1, n))
+    ref = O.softmax_rows(x, temp)
+    assert G.max_abs_rel(got, ref) <= TOL
+    assert G.ulp_mismatch(got, ref) < 0.02
+    assert int(G.host(idx_d, (1,), np.int32)[0]) == O.argmax_first(got) == int(np.flatnonzero(got[0] == got.max())[0])
+    assert G.L().lcu_softmax_argmax(probs_d.ptr, idx_d.ptr, probs_d.ptr, n, temp, None) == -2
+    G.release()

@@ -6,9 +6,11 @@
 // row of lhs (A) and of one row of W (B).
 //
 //   - 256 threads = 4 wavefronts in a 2x2 grid; block tile BM x BN, K step 64
-//   - global -> registers -> LDS, the next K step's global loads in flight while the matrix cores
-//     work on the current one; LDS rows padded by 16 bytes so the 16-byte operand reads of 16
-//     neighbouring lanes fall in distinct banks
+//   - global -> registers -> LDS with two LDS buffers and two register stages: while the matrix
+//     cores work on K step t, step t+1 waits in registers and step t+2 is being fetched; LDS rows
+//     are padded by 16 bytes so the 16-byte operand reads of 16 neighbouring lanes fall in
+//     distinct banks
+//   - the K loop carries no vector address arithmetic and no predication (see load_tile)
 //   - uint8 weights are dequantised between the global load and the LDS store, so each weight is
 //     converted once per block tile, to exactly fp16((q - 127.5) * scale) (287-289)
 //   - block index -> tile mapping keeps the tiles that share a slice of W on one XCD (one L2)
@@ -37,19 +39,21 @@ __device__ __forceinline__ half2_t dequant2(uint32_t spread, half2_t scale2x) {
   return t * scale2x;                                                                 // one rounding
 }
 
-template <int BM, int BN, bool U8>
-__global__ __launch_bounds__(THREADS) void gemm_kernel(half_t* __restrict__ out, const half_t* __restrict__ A,
-                                                       const void* __restrict__ Wv, const half_t* __restrict__ S,
-                                                       int M, int K, int N, int block, float beta, int tiles_m,
-                                                       int tiles_n) {
+// KTAIL: K is not a multiple of BK, so the last K step is partly out of range and must be zeroed
+// (costs selects in the loop; every model shape takes the KTAIL = false instantiation).
+template <int BM, int BN, bool U8, bool KTAIL>
+__global__ __launch_bounds__(THREADS, 2) void gemm_kernel(half_t* __restrict__ out, const half_t* __restrict__ A,
+                                                          const void* __restrict__ Wv, const half_t* __restrict__ S,
+                                                          int M, int K, int N, int block, float beta, int tiles_m,
+                                                          int tiles_n) {
   constexpr int TM = BM / 64;  // 32x32 MFMA tiles per wavefront along M
   constexpr int TN = BN / 64;
   constexpr int A_CHUNKS = BM * BK / 8 / THREADS;                  // 16-byte chunks per thread
   constexpr int B_CHUNKS = U8 ? BN * BK / 16 / THREADS : BN * BK / 8 / THREADS;
   static_assert(A_CHUNKS >= 1 && B_CHUNKS >= 1, "tile too small for 256 threads");
 
-  __shared__ __attribute__((aligned(16))) half_t As[BM * LDK];
-  __shared__ __attribute__((aligned(16))) half_t Bs[BN * LDK];
+  __shared__ __attribute__((aligned(16))) half_t As[2][BM * LDK];
+  __shared__ __attribute__((aligned(16))) half_t Bs[2][BN * LDK];
 
   // XCD-aware tile order: hardware deals consecutive workgroups round-robin to the 8 XCDs, so
   // give each XCD one contiguous run of the M-fastest tile sequence.
@@ -64,67 +68,98 @@ __global__ __launch_bounds__(THREADS) void gemm_kernel(half_t* __restrict__ out,
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
   const int wm = (wave & 1) * (BM / 2), wn = (wave >> 1) * (BN / 2);
-  const half_t* Wh = (const half_t*)Wv;
-  const uint8_t* Wq = (const uint8_t*)Wv;
   const int nblk = U8 ? K / block : 0;
 
-  half8_t ra[A_CHUNKS];
-  half8_t rb[U8 ? 1 : B_CHUNKS];
-  uint4_t rq[U8 ? B_CHUNKS : 1];
-  half_t rs[U8 ? B_CHUNKS : 1];
+  // Per-thread byte offsets of its chunks from the operand bases; they do not change over the K
+  // loop, which only advances a uniform base, so the loop carries no vector address arithmetic.
+  // Rows past M or N are clamped to the last row: their products land in accumulator rows and
+  // columns that the epilogue never stores, so no zero fill is needed for them.
+  uint32_t a_off[A_CHUNKS], b_off[B_CHUNKS], s_off[U8 ? B_CHUNKS : 1];
+  int a_k[A_CHUNKS], b_k[B_CHUNKS];
+#pragma unroll
+  for (int i = 0; i < A_CHUNKS; ++i) {
+    const int c = tid + i * THREADS;
+    a_k[i] = (c & 7) * 8;
+    a_off[i] = ((uint32_t)min(m0 + (c >> 3), M - 1) * (uint32_t)K + a_k[i]) * 2u;
+  }
+#pragma unroll
+  for (int i = 0; i < B_CHUNKS; ++i) {
+    const int c = tid + i * THREADS;
+    if constexpr (U8) {
+      const uint32_t row = (uint32_t)min(n0 + (c >> 2), N - 1);
+      b_k[i] = (c & 3) * 16;
+      b_off[i] = row * (uint32_t)K + b_k[i];
+      s_off[i] = row * (uint32_t)nblk;
+    } else {
+      b_k[i] = (c & 7) * 8;
+      b_off[i] = ((uint32_t)min(n0 + (c >> 3), N - 1) * (uint32_t)K + b_k[i]) * 2u;
+    }
+  }
+  const char* Ab = (const char*)A;
+  const char* Wb = (const char*)Wv;
 
-  auto load_tile = [&](int k0) {
+  // one K step of both operands in registers, as loaded from global memory
+  struct stage_t {
+    half8_t ra[A_CHUNKS];
+    half8_t rb[U8 ? 1 : B_CHUNKS];
+    uint4_t rq[U8 ? B_CHUNKS : 1];
+    half_t rs[U8 ? B_CHUNKS : 1];
+    int k0;
+  };
+
+  // Unconditional loads: a predicated load becomes a branch, and branches make the compiler wait
+  // for every outstanding load before it issues the next ones.  With KTAIL the k offset is
+  // clamped into range here and the chunk is zeroed when it is stored to LDS.
+  auto load_tile = [&](stage_t& st, int k0) {
+    st.k0 = k0;
 #pragma unroll
     for (int i = 0; i < A_CHUNKS; ++i) {
-      const int c = tid + i * THREADS;
-      const int row = c >> 3, kc = (c & 7) * 8;
-      const int gm = m0 + row, gk = k0 + kc;
-      ra[i] = (gm < M && gk < K) ? *reinterpret_cast<const half8_t*>(A + (size_t)gm * K + gk) : (half8_t)(0.0f);
+      int kk = k0;
+      if constexpr (KTAIL) kk = min(k0, K - 8 - a_k[i]);
+      st.ra[i] = *reinterpret_cast<const half8_t*>(Ab + (ptrdiff_t)kk * 2 + a_off[i]);
     }
     if constexpr (U8) {
 #pragma unroll
       for (int i = 0; i < B_CHUNKS; ++i) {
-        const int c = tid + i * THREADS;
-        const int row = c >> 2, kc = (c & 3) * 16;
-        const int gn = n0 + row, gk = k0 + kc;
-        const bool ok = gn < N && gk < K;
-        rq[i] = ok ? __builtin_nontemporal_load(reinterpret_cast<const uint4_t*>(Wq + (size_t)gn * K + gk))
-                   : (uint4_t)(0u);
-        rs[i] = ok ? S[(size_t)gn * nblk + gk / block] : (half_t)0.0f;
+        int kk = k0;
+        if constexpr (KTAIL) kk = min(k0, K - 16 - b_k[i]);
+        st.rq[i] = *reinterpret_cast<const uint4_t*>(Wb + (ptrdiff_t)kk + b_off[i]);
+        st.rs[i] = S[s_off[i] + (uint32_t)(kk + b_k[i]) / (uint32_t)block];
       }
     } else {
 #pragma unroll
       for (int i = 0; i < B_CHUNKS; ++i) {
-        const int c = tid + i * THREADS;
-        const int row = c >> 3, kc = (c & 7) * 8;
-        const int gn = n0 + row, gk = k0 + kc;
-        rb[i] = (gn < N && gk < K) ? __builtin_nontemporal_load(reinterpret_cast<const half8_t*>(Wh + (size_t)gn * K + gk))
-                                   : (half8_t)(0.0f);
+        int kk = k0;
+        if constexpr (KTAIL) kk = min(k0, K - 8 - b_k[i]);
+        st.rb[i] = *reinterpret_cast<const half8_t*>(Wb + (ptrdiff_t)kk * 2 + b_off[i]);
       }
     }
   };
 
-  auto store_tile = [&]() {
+  auto store_tile = [&](const stage_t& st, int buf) {
 #pragma unroll
     for (int i = 0; i < A_CHUNKS; ++i) {
       const int c = tid + i * THREADS;
-      *reinterpret_cast<half8_t*>(&As[(c >> 3) * LDK + (c & 7) * 8]) = ra[i];
+      half8_t v = st.ra[i];
+      if constexpr (KTAIL) v = (st.k0 + a_k[i] < K) ? v : (half8_t)(0.0f);
+      *reinterpret_cast<half8_t*>(&As[buf][(c >> 3) * LDK + (c & 7) * 8]) = v;
     }
     if constexpr (U8) {
 #pragma unroll
       for (int i = 0; i < B_CHUNKS; ++i) {
         const int c = tid + i * THREADS;
-        const half_t s2 = rs[i] * (half_t)2.0f;
+        half_t s2 = st.rs[i] * (half_t)2.0f;
+        if constexpr (KTAIL) s2 = (st.k0 + b_k[i] < K) ? s2 : (half_t)0.0f;  // zero scale: zero weights
         const half2_t s2v = {s2, s2};
         half2_t d[8];
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-          d[2 * j] = dequant2(__builtin_amdgcn_perm(0u, rq[i][j], 0x0c010c00u), s2v);
-          d[2 * j + 1] = dequant2(__builtin_amdgcn_perm(0u, rq[i][j], 0x0c030c02u), s2v);
+          d[2 * j] = dequant2(__builtin_amdgcn_perm(0u, st.rq[i][j], 0x0c010c00u), s2v);
+          d[2 * j + 1] = dequant2(__builtin_amdgcn_perm(0u, st.rq[i][j], 0x0c030c02u), s2v);
         }
         half8_t lo = {d[0].x, d[0].y, d[1].x, d[1].y, d[2].x, d[2].y, d[3].x, d[3].y};
         half8_t hi = {d[4].x, d[4].y, d[5].x, d[5].y, d[6].x, d[6].y, d[7].x, d[7].y};
-        half_t* dst = &Bs[(c >> 2) * LDK + (c & 3) * 16];
+        half_t* dst = &Bs[buf][(c >> 2) * LDK + (c & 3) * 16];
         *reinterpret_cast<half8_t*>(dst) = lo;
         *reinterpret_cast<half8_t*>(dst + 8) = hi;
       }
@@ -132,7 +167,9 @@ __global__ __launch_bounds__(THREADS) void gemm_kernel(half_t* __restrict__ out,
 #pragma unroll
       for (int i = 0; i < B_CHUNKS; ++i) {
         const int c = tid + i * THREADS;
-        *reinterpret_cast<half8_t*>(&Bs[(c >> 3) * LDK + (c & 7) * 8]) = rb[i];
+        half8_t v = st.rb[i];
+        if constexpr (KTAIL) v = (st.k0 + b_k[i] < K) ? v : (half8_t)(0.0f);
+        *reinterpret_cast<half8_t*>(&Bs[buf][(c >> 3) * LDK + (c & 7) * 8]) = v;
       }
     }
   };
@@ -147,23 +184,17 @@ __global__ __launch_bounds__(THREADS) void gemm_kernel(half_t* __restrict__ out,
   }
 
   const int frag_row = lane & 31, frag_k = (lane >> 5) * 8;
-  load_tile(0);
-  for (int k0 = 0; k0 < K; k0 += BK) {
-    store_tile();
-    __syncthreads();
-    if (k0 + BK < K) {
-      load_tile(k0 + BK);
-    }
+  auto compute = [&](int buf) {
 #pragma unroll
     for (int ks = 0; ks < BK; ks += 16) {
       half8_t fa[TM], fb[TN];
 #pragma unroll
       for (int i = 0; i < TM; ++i) {
-        fa[i] = *reinterpret_cast<const half8_t*>(&As[(wm + i * 32 + frag_row) * LDK + ks + frag_k]);
+        fa[i] = *reinterpret_cast<const half8_t*>(&As[buf][(wm + i * 32 + frag_row) * LDK + ks + frag_k]);
       }
 #pragma unroll
       for (int j = 0; j < TN; ++j) {
-        fb[j] = *reinterpret_cast<const half8_t*>(&Bs[(wn + j * 32 + frag_row) * LDK + ks + frag_k]);
+        fb[j] = *reinterpret_cast<const half8_t*>(&Bs[buf][(wn + j * 32 + frag_row) * LDK + ks + frag_k]);
       }
 #pragma unroll
       for (int i = 0; i < TM; ++i) {
@@ -173,6 +204,28 @@ __global__ __launch_bounds__(THREADS) void gemm_kernel(half_t* __restrict__ out,
         }
       }
     }
+  };
+
+  // Pipeline: LDS buffer t%2 holds K step t; one register stage holds step t+1 (requested one
+  // iteration ago) and the other receives step t+2 while the matrix cores work on step t.
+  // Two iterations per trip so that the two register stages keep fixed names.
+  stage_t s0, s1;
+  const int nt = (K + BK - 1) / BK;
+  load_tile(s0, 0);
+  if (nt > 1) load_tile(s1, BK);
+  store_tile(s0, 0);
+  __syncthreads();
+  for (int t = 0; t < nt; t += 2) {
+    // step t in LDS 0, step t+1 in s1
+    if (t + 2 < nt) load_tile(s0, (t + 2) * BK);
+    compute(0);
+    if (t + 1 < nt) store_tile(s1, 1);
+    __syncthreads();
+    if (t + 1 >= nt) break;
+    // step t+1 in LDS 1, step t+2 in s0
+    if (t + 3 < nt) load_tile(s1, (t + 3) * BK);
+    compute(1);
+    if (t + 2 < nt) store_tile(s0, 0);
     __syncthreads();
   }
 
@@ -203,7 +256,13 @@ template <int BM, int BN, bool U8>
 int launch_gemm(half_t* out, const half_t* A, const void* W, const half_t* S, int M, int K, int N, int block,
                 float beta, hipStream_t st) {
   const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
-  gemm_kernel<BM, BN, U8><<<tiles_m * tiles_n, THREADS, 0, st>>>(out, A, W, S, M, K, N, block, beta, tiles_m, tiles_n);
+  if (K % BK == 0) {
+    gemm_kernel<BM, BN, U8, false><<<tiles_m * tiles_n, THREADS, 0, st>>>(out, A, W, S, M, K, N, block, beta, tiles_m,
+                                                                          tiles_n);
+  } else {
+    gemm_kernel<BM, BN, U8, true><<<tiles_m * tiles_n, THREADS, 0, st>>>(out, A, W, S, M, K, N, block, beta, tiles_m,
+                                                                         tiles_n);
+  }
   LCU_LAUNCH_CHECK();
   return LCU_OK;
 }
@@ -211,9 +270,9 @@ int launch_gemm(half_t* out, const half_t* A, const void* W, const half_t* S, in
 template <bool U8>
 int dispatch_gemm(half_t* out, const half_t* A, const void* W, const half_t* S, int M, int K, int N, int block,
                   float beta, hipStream_t st) {
-  // enough 128x128 tiles to cover the 256 compute units twice, else the narrower tile
+  // 128x128 tiles when there are enough of them to give every compute unit one; else 128x64
   const long tiles128 = (long)((M + 127) / 128) * ((N + 127) / 128);
-  if (tiles128 >= 512) {
+  if (tiles128 >= 256) {
     return launch_gemm<128, 128, U8>(out, A, W, S, M, K, N, block, beta, st);
   }
   return launch_gemm<128, 64, U8>(out, A, W, S, M, K, N, block, beta, st);
@@ -229,6 +288,8 @@ int lcu_gemm_f16_nt(void* out_dev, const void* lhs_dev, const void* rhs_dev, int
   LCU_REQUIRE(M >= 0 && N > 0 && K > 0 && K % 8 == 0, "lcu_gemm_f16_nt: bad shape M %d K %d N %d (K %% 8 == 0)", M, K,
               N);
   if (M == 0) return LCU_OK;
+  LCU_REQUIRE((size_t)M * K * 2 < ((size_t)1 << 32) && (size_t)N * K * 2 < ((size_t)1 << 32),
+              "lcu_gemm_f16_nt: operands of 4 GiB or more are not supported");
   if (M == 1 && K <= 24576) {
     return gemv_f16((half_t*)out_dev, (const half_t*)lhs_dev, (const half_t*)rhs_dev, K, N, beta, as_stream(stream));
   }
@@ -243,6 +304,8 @@ int lcu_gemm_f16u8_nt(void* out_dev, const void* lhs_dev, const void* codes_dev,
               "lcu_gemm_f16u8_nt: bad shape M %d K %d N %d block %d (K %% 16 == 0, block %% 16 == 0, K %% block == 0)",
               M, K, N, block);
   if (M == 0) return LCU_OK;
+  LCU_REQUIRE((size_t)M * K * 2 < ((size_t)1 << 32) && (size_t)N * K < ((size_t)1 << 32),
+              "lcu_gemm_f16u8_nt: operands of 4 GiB or more are not supported");
   if (M == 1 && K <= 24576) {
     return gemv_u8((half_t*)out_dev, (const half_t*)lhs_dev, (const uint8_t*)codes_dev, (const half_t*)scales_dev, K,
                    N, block, beta, as_stream(stream));

@@ -152,6 +152,16 @@ def test_one_llama7b_layer_prefill_512_then_decode_at_2048(gpu):
     assert G.max_abs_rel(gk, ok) <= TOL and G.max_abs_rel(gv, ov) <= TOL
 
 
+# Greedy decoding compares argmax results, and an argmax is discontinuous: where the oracle's two
+# largest fp16 logits are within a few fp16 ulps of each other (logits of 4..8 have an ulp of
+# 0.0039), any other correct fp32-accumulating implementation -- the reference's own matmul_type 1
+# versus 4 included -- may order them the other way.  So every step must reproduce the oracle's
+# token, except at steps whose oracle margin is at most NEAR_TIE, where the device must still pick
+# one of the oracle's two candidates.  Steps are compared under teacher forcing (the oracle's token
+# is fed back), so one near-tie cannot hide the steps after it.
+NEAR_TIE = 0.02
+
+
 def greedy_case(G, name):
     path = os.path.join(GOLDEN, name)
     if not os.path.exists(path):
@@ -162,27 +172,36 @@ def greedy_case(G, name):
                    seed=fx["seed"], weight_std=fx["weight_std"])
     gc = G.P.Context(gm, context_len=fx["context_len"], temperature=fx["temperature"])
     feed = np.array(fx["prompt"], dtype=np.int16)
-    got, report = [], []
+    identical, near_ties, failures = 0, [], []
     for step, want in enumerate(fx["tokens"]):
         tok = gc.next_token(feed)
-        got.append(tok)
-        if tok != want:
-            l1, l2, p1, p2 = fx["top2_logits_probs"][step]
-            report.append("step %d: device %d, oracle %d; oracle top-2 logits %.5f / %.5f (margin %.5f)"
-                          % (step, tok, want, l1, l2, l1 - l2))
-        feed = np.array([want], dtype=np.int16)  # teacher forcing: every step is compared on the oracle's sequence
+        l1, l2, _, _ = fx["top2_logits_probs"][step]
+        if tok == want:
+            identical += 1
+        elif l1 - l2 <= NEAR_TIE and tok in fx["top2_ids"][step]:
+            near_ties.append("step %d: device %d, oracle %d; oracle top-2 logits %.5f / %.5f" % (step, tok, want, l1, l2))
+        else:
+            failures.append("step %d: device %d, oracle %d (top-2 ids %s); oracle top-2 logits %.5f / %.5f"
+                            % (step, tok, want, fx["top2_ids"][step], l1, l2))
+        feed = np.array([want], dtype=np.int16)
     gc.close()
     gm.close()
-    return got, fx["tokens"], report
+    print("%s: %d of %d steps identical; near-tie steps: %s" % (name, identical, len(fx["tokens"]), near_ties or "none"))
+    n_close = sum(1 for t in fx["top2_logits_probs"] if t[0] - t[1] <= NEAR_TIE)
+    return identical, len(fx["tokens"]), near_ties, failures, n_close
 
 
 def test_greedy_tokens_llama7b_fp16(gpu):
-    """Full LLaMA-7B shape, fp16: 512-token prompt, 128 greedy steps identical to the oracle's."""
-    got, want, report = greedy_case(gpu, "llama7b_fp16_seed0_greedy.json")
-    assert got == want, "\n".join(report)
+    """Full LLaMA-7B shape, fp16, 512-token prompt, 128 greedy steps against the oracle's tokens."""
+    identical, total, near_ties, failures, n_close = greedy_case(gpu, "llama7b_fp16_seed0_greedy.json")
+    assert not failures, "\n".join(failures)
+    assert identical + len(near_ties) == total and len(near_ties) <= n_close
+    assert identical >= total - 4
 
 
 def test_greedy_tokens_llama30b_u8(gpu):
-    """LLaMA-30B shape, uint8 weights: 512-token prompt, 128 greedy steps identical to the oracle's."""
-    got, want, report = greedy_case(gpu, "llama30b_u8_seed0_greedy.json")
-    assert got == want, "\n".join(report)
+    """LLaMA-30B shape, uint8 weights, 512-token prompt, 128 greedy steps against the oracle's tokens."""
+    identical, total, near_ties, failures, n_close = greedy_case(gpu, "llama30b_u8_seed0_greedy.json")
+    assert not failures, "\n".join(failures)
+    assert identical + len(near_ties) == total and len(near_ties) <= n_close
+    assert identical >= total - 4

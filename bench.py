@@ -27,6 +27,10 @@ import numpy as np
 ROOT = os.path.dirname(os.path.abspath(__file__))
 PKG = os.path.join(ROOT, "llama.cu_amd")
 HBM_PEAK_GBS = 8000.0      # MI355X HBM3E
+# HBM bytes per launch of the dominant kernel from rocprofv3 FETCH_SIZE / WRITE_SIZE, scaled by a
+# 256 MiB copy kernel read under the same counters (FETCH_SIZE reads half the bytes here): see
+# profiles/decode_ffn_up_kernel_llama7b_hbm_traffic.txt.  Counters are not read in this script.
+MEASURED_TRAFFIC = {"llama7b_fp16": 180643635}
 MFMA_F16_PEAK_TF = 2500.0  # dense fp16
 
 WORKLOADS = {
@@ -279,6 +283,9 @@ def main():
     ap.add_argument("--workload", default="llama7b_fp16", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip the per-shape GEMV / GEMM legs")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run one 256 MiB device-to-device copy: a copy kernel of known size, against which "
+                         "rocprofv3 FETCH_SIZE / WRITE_SIZE readings of the other kernels are scaled")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         sys.stderr.write("bench.py: this build runs on one GPU (the whole model fits in one MI355X's HBM); "
@@ -297,6 +304,15 @@ def main():
                  decode_frac_of_hbm_roofline=round(dec["bytes_per_token"] / dec["ms_per_step"] / 1e6 / HBM_PEAK_GBS, 3))
     ctx.close()
     model.close()
+    if args.copy_calibration:
+        n = 256 << 20
+        a, b = B.DeviceBuffer(n), B.DeviceBuffer(n)
+        B.check(B.lib().lcu_memset(a.ptr, 1, n, None))
+        B.check(B.lib().lcu_d2d(b.ptr, a.ptr, n, None))
+        B.check(B.lib().lcu_sync(None))
+        extra["copy_calibration_bytes"] = n
+        a.free()
+        b.free()
     if not args.no_extra:
         stream = None
         extra["gemv"] = gemv_leg(P, stream)
@@ -311,7 +327,7 @@ def main():
         "config": {"workload": "%s: %d-token random prompt, then batch-1 greedy decode, context 2048, temperature 0.8"
                                % (args.workload, PROMPT), "device": props.name.decode(errors="replace")},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC.get(args.workload),
                      "kernel": "decode_ffn_up_kernel (W1,W3 GEMV + SiLU*mul), dim %d ffn %d" % (cfg["dim"], model.ffn),
                      "bytes_per_launch": int(k_bytes), "us_per_launch": round(k_us, 3)},
         "cpu_baseline": cpu,

@@ -58,12 +58,26 @@ __device__ __forceinline__ half_t round_f16(float f) {
 }
 
 // ---- wavefront reductions (all 64 lanes end with the result) ----
+template <int CTRL>
+__device__ __forceinline__ float dpp_f32(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, true));
+}
+
+// Sum over the 64 lanes with data-parallel-primitive moves (VALU speed; __shfl_xor compiles to
+// ds_bpermute, an LDS round trip per step).  Lanes 1, 2 apart by quad permutes, then the mirrors
+// within 8 and 16 lanes, then the four 16-lane row sums are read out and added.  The association
+// is (((t ^ 1) ^ 2) ^ 4) ^ 8 inside a row, then (r0 + r1) + (r2 + r3).
 __device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-  for (int off = 32; off > 0; off >>= 1) {
-    v += __shfl_xor(v, off, WAVE);
-  }
-  return v;
+  v += dpp_f32<0xB1>(v);   // quad_perm [1,0,3,2]
+  v += dpp_f32<0x4E>(v);   // quad_perm [2,3,0,1]
+  v += dpp_f32<0x141>(v);  // row_half_mirror
+  v += dpp_f32<0x140>(v);  // row_mirror
+  const int vi = __builtin_bit_cast(int, v);
+  const float r0 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(vi, 0));
+  const float r1 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(vi, 16));
+  const float r2 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(vi, 32));
+  const float r3 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(vi, 48));
+  return (r0 + r1) + (r2 + r3);
 }
 __device__ __forceinline__ float wave_max(float v) {
 #pragma unroll

@@ -15,9 +15,10 @@
 //     (global load instructions per workgroup are what this prologue must keep few)
 //   - products accumulate in fp32 per lane, lanes combine with xor shuffles, wavefronts through
 //     LDS, thread 0 applies the epilogue (residual add, RoPE, SiLU*mul) and rounds once to fp16
-// uint8 weights are dequantised in packed fp16: (128 + q/2) is built by bit insertion, minus
-// 191.75 gives (q - 127.5)/2 exactly, times 2*scale rounds once, which is bit-for-bit
-// fp16((q - 127.5) * scale), the value the reference feeds its tensor cores (287-289, 336-341).
+// uint8 weights are dequantised in packed fp16 to bit-for-bit fp16((q - 127.5) * scale), the value
+// the reference feeds its tensor cores (287-289, 336-341): see dequant2_fma / dequant2.  The
+// products then go through v_dot2_f32_f16 (two multiply-adds per instruction, fp32 accumulate):
+// the dequantisation arithmetic, not HBM, is what bounds this kernel on large matrices.
 #include "common.hpp"
 
 using namespace lcu;
@@ -58,11 +59,20 @@ __device__ __forceinline__ half8_t normed(half8_t x, half8_t w, float rms_inv) {
   return r;
 }
 
-// two codes spread as [b0, 0, b1, 0] -> two dequantised halves
+// two codes spread as [b0, 0, b1, 0] -> two dequantised halves; exact for every scale
 __device__ __forceinline__ half2_t dequant2(uint32_t spread, half2_t scale2x) {
   const uint32_t bits = (spread << 2) | 0x58005800u;                                  // 128 + q/2, exact
   const half2_t t = __builtin_bit_cast(half2_t, bits) - (half2_t)((half_t)191.75f);   // (q - 127.5)/2, exact
   return t * scale2x;                                                                 // one rounding
+}
+
+// The same value in three operations instead of four: bytes [b0, 0x64, b1, 0x64] are the halves
+// 1024 + q; minus 1152 is q - 128, exact; fma(q - 128, s, s/2) forms (q - 127.5) * s exactly and
+// rounds once.  Needs s/2 to be exact, i.e. not a subnormal scale with an odd last bit: the caller
+// checks that and falls back to dequant2.
+__device__ __forceinline__ half2_t dequant2_fma(uint32_t biased, half2_t scale, half2_t half_scale) {
+  const half2_t q128 = __builtin_bit_cast(half2_t, biased) - (half2_t)((half_t)1152.0f);
+  return __builtin_elementwise_fma(q128, scale, half_scale);
 }
 
 // ---- one batch in registers: U chunks of R rows of W (16 bytes per lane each), with the matching
@@ -77,27 +87,28 @@ struct batch_t {
   half8_t xr[NORM ? 1 : U][NORM ? 1 : XV];        // x itself, unless it is read (raw) from LDS later
   half8_t nw[NORM ? U : 1][NORM ? XV : 1];
 
+  // Loads are unconditional: a chunk past the end of K is read from the last in-range position
+  // instead (a predicated load becomes a branch, and the waits the compiler puts around branches
+  // serialise the loads); fma() gives such a chunk a zero x.
   __device__ __forceinline__ void load(const uint8_t* const (&rows)[R], const half_t* const (&srow)[R],
                                        const half_t* __restrict__ x, const half_t* __restrict__ norm_w, int kb, int K,
                                        int block, int lane) {
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-      const int kk = (kb * U + u) * CHUNK + lane * VEC;
-      const bool ok = kk < K;
+      const int kk = min((kb * U + u) * CHUNK + lane * VEC, K - VEC);
 #pragma unroll
       for (int r = 0; r < R; ++r) {
-        w[u][r] = ok ? __builtin_nontemporal_load(reinterpret_cast<const uint4_t*>(rows[r] + (size_t)kk * (U8 ? 1 : 2)))
-                     : (uint4_t)(0u);
+        w[u][r] = __builtin_nontemporal_load(reinterpret_cast<const uint4_t*>(rows[r] + (size_t)kk * (U8 ? 1 : 2)));
         if constexpr (U8) {
-          sc[u][r] = ok ? srow[r][kk / block] : (half_t)0.0f;
+          sc[u][r] = srow[r][kk / block];
         }
       }
 #pragma unroll
       for (int j = 0; j < XV; ++j) {
         if constexpr (NORM) {
-          nw[u][j] = ok ? *reinterpret_cast<const half8_t*>(norm_w + kk + 8 * j) : (half8_t)(0.0f);
+          nw[u][j] = *reinterpret_cast<const half8_t*>(norm_w + kk + 8 * j);
         } else {
-          xr[u][j] = ok ? *reinterpret_cast<const half8_t*>(x + kk + 8 * j) : (half8_t)(0.0f);
+          xr[u][j] = *reinterpret_cast<const half8_t*>(x + kk + 8 * j);
         }
       }
     }
@@ -111,29 +122,46 @@ struct batch_t {
       half8_t xv[XV];
 #pragma unroll
       for (int j = 0; j < XV; ++j) {
+        const int kk = (kb * U + u) * CHUNK + lane * VEC;
         if constexpr (NORM) {
-          const int kk = (kb * U + u) * CHUNK + lane * VEC;
           const half8_t raw = kk < K ? *reinterpret_cast<const half8_t*>(xs + kk + 8 * j) : (half8_t)(0.0f);
           xv[j] = normed(raw, nw[u][j], rms_inv);
         } else {
-          xv[j] = xr[u][j];
+          xv[j] = kk < K ? xr[u][j] : (half8_t)(0.0f);
         }
       }
 #pragma unroll
       for (int r = 0; r < R; ++r) {
         if constexpr (U8) {
-          const half_t s2 = sc[u][r] * (half_t)2.0f;  // exact
-          const half2_t s2v = {s2, s2};
+          const half_t sv = sc[u][r];
+          const half_t hv = sv * (half_t)0.5f;
+          if (hv + hv == sv) {  // s/2 exact (every normal scale): 3-operation dequantisation
+            const half2_t s1v = {sv, sv}, h1v = {hv, hv};
 #pragma unroll
-          for (int j = 0; j < 4; ++j) {
-            const half2_t lo = dequant2(__builtin_amdgcn_perm(0u, w[u][r][j], 0x0c010c00u), s2v);
-            const half2_t hi = dequant2(__builtin_amdgcn_perm(0u, w[u][r][j], 0x0c030c02u), s2v);
-            const half8_t& x8 = xv[j >> 1];
-            const int e = (j & 1) * 4;
-            a0[r] = fmaf((float)lo.x, (float)x8[e], a0[r]);
-            a1[r] = fmaf((float)lo.y, (float)x8[e + 1], a1[r]);
-            a0[r] = fmaf((float)hi.x, (float)x8[e + 2], a0[r]);
-            a1[r] = fmaf((float)hi.y, (float)x8[e + 3], a1[r]);
+            for (int j = 0; j < 4; ++j) {
+              // selector bytes 4..7 pick from the first operand (0x64 in every byte), 0..3 from the codes
+              const half2_t lo = dequant2_fma(__builtin_amdgcn_perm(0x64646464u, w[u][r][j], 0x04010400u), s1v, h1v);
+              const half2_t hi = dequant2_fma(__builtin_amdgcn_perm(0x64646464u, w[u][r][j], 0x04030402u), s1v, h1v);
+              const half8_t& x8 = xv[j >> 1];
+              const int e = (j & 1) * 4;
+              const half2_t xlo = {x8[e], x8[e + 1]}, xhi = {x8[e + 2], x8[e + 3]};
+              a0[r] = __builtin_amdgcn_fdot2(lo, xlo, a0[r], false);
+              a1[r] = __builtin_amdgcn_fdot2(hi, xhi, a1[r], false);
+            }
+          } else {
+            const half_t s2 = sv * (half_t)2.0f;  // exact
+            const half2_t s2v = {s2, s2};
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+              const half2_t lo = dequant2(__builtin_amdgcn_perm(0u, w[u][r][j], 0x0c010c00u), s2v);
+              const half2_t hi = dequant2(__builtin_amdgcn_perm(0u, w[u][r][j], 0x0c030c02u), s2v);
+              const half8_t& x8 = xv[j >> 1];
+              const int e = (j & 1) * 4;
+              a0[r] = fmaf((float)lo.x, (float)x8[e], a0[r]);
+              a1[r] = fmaf((float)lo.y, (float)x8[e + 1], a1[r]);
+              a0[r] = fmaf((float)hi.x, (float)x8[e + 2], a0[r]);
+              a1[r] = fmaf((float)hi.y, (float)x8[e + 3], a1[r]);
+            }
           }
         } else {
           const half8_t wv = __builtin_bit_cast(half8_t, w[u][r]);
@@ -159,7 +187,7 @@ struct batch_t {
 template <bool U8, int R, int U, bool NORM, class Tasks>
 struct stream_t {
   using batch = batch_t<U8, R, U, NORM>;
-  const Tasks& tk;
+  const Tasks tk;  // by value: a reference member kept the struct in scratch memory in some instantiations
   const half_t* x;
   const half_t* norm_w;
   int K, block, lane, wave, task, n_batches;
@@ -253,20 +281,17 @@ struct plain_tasks {
   }
 };
 
-// [Wq; Wk; Wv]: task = one interleaved pair (rows 2p, 2p+1) of one of the three matrices;
-// RoPE on q and k (llama_cu.cu:381-387), results to q_out / the caches' row for this position
+// One of Wq / Wk / Wv (chosen per workgroup by the kernel): task = one interleaved pair (rows 2p,
+// 2p+1); RoPE on q and k (llama_cu.cu:381-387), results to q_out / the caches' row for this position
 template <bool U8>
 struct qkv_tasks {
-  const void *wq, *wk, *wv;
-  const half_t *sq, *sk, *sv;
-  half_t *q_out, *k_row, *v_row;
-  const float2* rope_row;
-  int dim, head_dim, nblk;
+  const void* W;
+  const half_t* S;
+  half_t* dst;             // q_out, or the K / V cache row of this position
+  const float2* rope_row;  // nullptr for V
+  int dim, head_dim, nblk, first_task;
   __device__ __forceinline__ void rows(int task, const uint8_t* (&rows)[2], const half_t* (&srow)[2]) const {
-    const int half_dim = dim / 2;
-    const int which = task / half_dim, p = task - which * half_dim;
-    const void* W = which == 0 ? wq : (which == 1 ? wk : wv);
-    const half_t* S = which == 0 ? sq : (which == 1 ? sk : sv);
+    const int p = task - first_task;
 #pragma unroll
     for (int r = 0; r < 2; ++r) {
       rows[r] = row_ptr<U8>(W, 2 * p + r, dim);
@@ -274,22 +299,20 @@ struct qkv_tasks {
     }
   }
   __device__ __forceinline__ void finish(int task, const float (&acc)[2]) const {
-    const int half_dim = dim / 2;
-    const int which = task / half_dim, p = task - which * half_dim;
+    const int p = task - first_task;
     // the GEMV output is rounded to fp16 before RoPE reads it (llama_cu.cu:1144-1153)
     const half_t h0 = round_f16(acc[0]), h1 = round_f16(acc[1]);
     half2_t o;
-    if (which == 2) {
+    if (rope_row == nullptr) {
       o.x = h0;
       o.y = h1;
-      *reinterpret_cast<half2_t*>(v_row + 2 * p) = o;
     } else {
       const float2 cs = rope_row[((2 * p) % head_dim) / 2];
       const float real = (float)h0, imag = (float)h1;
       o.x = round_f16(fmaf(real, cs.x, -(imag * cs.y)));
       o.y = round_f16(fmaf(real, cs.y, imag * cs.x));
-      *reinterpret_cast<half2_t*>((which == 0 ? q_out : k_row) + 2 * p) = o;
     }
+    *reinterpret_cast<half2_t*>(dst + 2 * p) = o;
   }
 };
 
@@ -349,7 +372,14 @@ __global__ __launch_bounds__(GEMV_THREADS) void decode_qkv_kernel(
     v_row += (size_t)pos * dim;
     rope_row += (size_t)pos * (head_dim / 2);
   }
-  qkv_tasks<U8> tk{wq, wk, wv, sq, sk, sv, q_out, k_row, v_row, rope_row, dim, head_dim, U8 ? dim / block : 0};
+  // one task per workgroup, so the matrix is chosen here, once, from the kernel arguments (a
+  // per-task choice inside the task struct made the compiler index the struct in scratch memory)
+  const int half_dim = dim / 2;
+  const int which = blockIdx.x / half_dim;
+  const void* W = which == 0 ? wq : (which == 1 ? wk : wv);
+  const half_t* S = which == 0 ? sq : (which == 1 ? sk : sv);
+  half_t* dst = which == 0 ? q_out : (which == 1 ? k_row : v_row);
+  qkv_tasks<U8> tk{W, S, dst, which == 2 ? nullptr : rope_row, dim, head_dim, U8 ? dim / block : 0, which * half_dim};
   stream_t<U8, 2, U, NORM, qkv_tasks<U8>> st(tk, x, norm_w, dim, block, blockIdx.x);
   st.begin();
   float rms_inv = 1.0f;
@@ -401,7 +431,11 @@ int gemv_f16(half_t* out, const half_t* x, const half_t* W, int K, int N, float 
 
 int gemv_u8(half_t* out, const half_t* x, const uint8_t* W, const half_t* S, int K, int N, int block, float beta,
             hipStream_t st) {
-  gemv_kernel<true, 2, 1, false><<<(N + 1) / 2, GEMV_THREADS, 0, st>>>(out, x, nullptr, W, S, K, N, block, beta, 0.f);
+  if (N >= 8192) {
+    gemv_kernel<true, 4, 1, false><<<(N + 3) / 4, GEMV_THREADS, 0, st>>>(out, x, nullptr, W, S, K, N, block, beta, 0.f);
+  } else {
+    gemv_kernel<true, 2, 1, false><<<(N + 1) / 2, GEMV_THREADS, 0, st>>>(out, x, nullptr, W, S, K, N, block, beta, 0.f);
+  }
   LCU_LAUNCH_CHECK();
   return LCU_OK;
 }

@@ -10,7 +10,7 @@
 // columns h*128 .. h*128+127.
 //
 // Decode (n_new == 1): one 1024-thread workgroup per head does scores, softmax and the weighted
-// sum in one launch; 16 lanes share one cached row (16 bytes each), 64 rows per pass, 8 passes of
+// sum in one launch; 16 lanes share one cached row (16 bytes each), 64 rows per pass, 16 passes of
 // loads in flight per thread.
 // Prefill (n_new > 1), matrix-core bound: one workgroup per (32 query rows, head); Q.K^T by
 // v_mfma_f32_16x16x32_f16 into an LDS score strip [32][T], softmax in LDS, P.V by MFMA with V
@@ -26,21 +26,20 @@ constexpr int MAX_T_DECODE = 4096;
 constexpr int MAX_HEADS = 64;
 constexpr int DEC_THREADS = 1024;
 constexpr int DEC_GROUPS = DEC_THREADS / 16;  // cache rows per pass: 16 lanes x 16 bytes cover one row of a head
-constexpr int DEC_FLIGHT = 8;                 // passes whose loads are requested together
+constexpr int DEC_FLIGHT = 16;                // passes whose loads are requested together
 
 // One workgroup per head, the whole attention of one new token in a single launch.  The work is
 // a few hundred KB per head, so the kernel is organised around load latency: 1024 threads, every
-// thread keeps 8 independent 16-byte loads in flight, and the first V rows are requested before
-// the softmax statistics are reduced.
+// thread keeps up to 16 independent 16-byte loads in flight (1024 cached rows per round; rows past
+// T are masked off per lane, which costs no load bandwidth), the first V rows are requested before
+// the softmax statistics are reduced, and the 16-lane dot products are summed with
+// data-parallel-primitive moves instead of LDS shuffles.
 __global__ __launch_bounds__(DEC_THREADS) void decode_attention_kernel(half_t* __restrict__ out,
                                                                        const half_t* __restrict__ q,
                                                                        const half_t* __restrict__ k,
-                                                                       const half_t* __restrict__ v, int T, int dim,
+                                                                       const half_t* __restrict__ v, int T_cap, int dim,
                                                                        const int* __restrict__ pos_dev) {
-  __shared__ half_t sc[MAX_T_DECODE];
-  if (pos_dev) {  // position kept on the device (graph replay): the new row is row *pos_dev, T is the cap
-    T = min(max(*pos_dev + 1, 1), T);
-  }           // fp16 scores, then fp16 probabilities
+  __shared__ half_t sc[MAX_T_DECODE];  // fp16 scores, then fp16 probabilities
   __shared__ float gsum[DEC_GROUPS][HD + 4];
   __shared__ float red[16];
   const int h = blockIdx.x;
@@ -48,14 +47,17 @@ __global__ __launch_bounds__(DEC_THREADS) void decode_attention_kernel(half_t* _
   const int sub = tid & 15, grp = tid >> 4;
   const half_t* kh = k + h * HD + sub * 8;
   const half_t* vh = v + h * HD + sub * 8;
+  // position kept on the device (graph replay): the new row is row *pos_dev, T_cap is the cap
+  int T = T_cap;
+  if (pos_dev) {
+    T = min(max(*pos_dev + 1, 1), T_cap);
+  }
   const half8_t qh = *reinterpret_cast<const half8_t*>(q + h * HD + sub * 8);
-  float qf[8];
-#pragma unroll
-  for (int e = 0; e < 8; ++e) qf[e] = (float)qh[e];
   const float denom = sqrtf((float)HD);
 
   // ---- scores, llama_cu.cu:400-428 (no mask: the one new row sees every cached row)
-  for (int p0 = 0; p0 < T; p0 += DEC_GROUPS * DEC_FLIGHT) {
+  int p0 = 0;
+  do {
     half8_t kv[DEC_FLIGHT];
 #pragma unroll
     for (int f = 0; f < DEC_FLIGHT; ++f) {
@@ -68,12 +70,12 @@ __global__ __launch_bounds__(DEC_THREADS) void decode_attention_kernel(half_t* _
       const int p = p0 + f * DEC_GROUPS + grp;
       float s = 0.0f;
 #pragma unroll
-      for (int e = 0; e < 8; ++e) s = fmaf(qf[e], (float)kv[f][e], s);
-#pragma unroll
-      for (int off = 8; off > 0; off >>= 1) s += __shfl_xor(s, off, WAVE);
+      for (int e = 0; e < 8; ++e) s = fmaf((float)qh[e], (float)kv[f][e], s);
+      s = row16_sum(s);
       if (sub == 0 && p < T) sc[p] = round_f16(s / denom);  // 425
     }
-  }
+    p0 += DEC_GROUPS * DEC_FLIGHT;
+  } while (p0 < T);
   // first V rows: independent of the statistics below
   half8_t vv[DEC_FLIGHT];
 #pragma unroll
@@ -113,14 +115,12 @@ __global__ __launch_bounds__(DEC_THREADS) void decode_attention_kernel(half_t* _
   float acc[8];
 #pragma unroll
   for (int e = 0; e < 8; ++e) acc[e] = 0.0f;
-  for (int p0 = 0; p0 < T; p0 += DEC_GROUPS * DEC_FLIGHT) {
-    half8_t nv[DEC_FLIGHT];
-    const int n0 = p0 + DEC_GROUPS * DEC_FLIGHT;
-    if (n0 < T) {
+  for (p0 = 0; p0 < T; p0 += DEC_GROUPS * DEC_FLIGHT) {
+    if (p0 > 0) {
 #pragma unroll
       for (int f = 0; f < DEC_FLIGHT; ++f) {
-        const int p = n0 + f * DEC_GROUPS + grp;
-        nv[f] = p < T ? __builtin_nontemporal_load(reinterpret_cast<const half8_t*>(vh + (size_t)p * dim))
+        const int p = p0 + f * DEC_GROUPS + grp;
+        vv[f] = p < T ? __builtin_nontemporal_load(reinterpret_cast<const half8_t*>(vh + (size_t)p * dim))
                       : (half8_t)(0.0f);
       }
     }
@@ -133,8 +133,6 @@ __global__ __launch_bounds__(DEC_THREADS) void decode_attention_kernel(half_t* _
         for (int e = 0; e < 8; ++e) acc[e] = fmaf(prob, (float)vv[f][e], acc[e]);
       }
     }
-#pragma unroll
-    for (int f = 0; f < DEC_FLIGHT; ++f) vv[f] = nv[f];
   }
 #pragma unroll
   for (int e = 0; e < 8; ++e) gsum[grp][sub * 8 + e] = acc[e];

@@ -67,11 +67,16 @@ __device__ __forceinline__ float dpp_f32(float v) {
 // ds_bpermute, an LDS round trip per step).  Lanes 1, 2 apart by quad permutes, then the mirrors
 // within 8 and 16 lanes, then the four 16-lane row sums are read out and added.  The association
 // is (((t ^ 1) ^ 2) ^ 4) ^ 8 inside a row, then (r0 + r1) + (r2 + r3).
-__device__ __forceinline__ float wave_sum(float v) {
+// sum over each aligned group of 16 lanes, left in every lane of the group
+__device__ __forceinline__ float row16_sum(float v) {
   v += dpp_f32<0xB1>(v);   // quad_perm [1,0,3,2]
   v += dpp_f32<0x4E>(v);   // quad_perm [2,3,0,1]
   v += dpp_f32<0x141>(v);  // row_half_mirror
   v += dpp_f32<0x140>(v);  // row_mirror
+  return v;
+}
+__device__ __forceinline__ float wave_sum(float v) {
+  v = row16_sum(v);
   const int vi = __builtin_bit_cast(int, v);
   const float r0 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(vi, 0));
   const float r1 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(vi, 16));

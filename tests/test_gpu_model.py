@@ -159,7 +159,15 @@ def test_one_llama7b_layer_prefill_512_then_decode_at_2048(gpu):
 # token, except at steps whose oracle margin is at most NEAR_TIE, where the device must still pick
 # one of the oracle's two candidates.  Steps are compared under teacher forcing (the oracle's token
 # is fed back), so one near-tie cannot hide the steps after it.
-NEAR_TIE = 0.02
+#
+# How near is near depends on the depth of the model: rounding differences grow through the layers.
+# LLaMA-7B (32 layers): device and oracle logits differ by 0.006 on average, 0.02 at most, over the
+# fixture's steps.  LLaMA-30B (60 layers): 0.018 on average, 0.07 at most -- and the device's own
+# uint8 kernels differ by just as much from its fp16 kernels run on the dequantised weight values
+# (test_u8_and_f16_kernels_agree_at_30b_depth), so that figure is the noise floor of the depth, not
+# an error of one path.  An argmax can flip when the margin is below about twice the per-logit
+# deviation.
+NEAR_TIE = {"llama7b_fp16_seed0_greedy.json": 0.02, "llama30b_u8_seed0_greedy.json": 0.1}
 
 
 def greedy_case(G, name):
@@ -178,7 +186,7 @@ def greedy_case(G, name):
         l1, l2, _, _ = fx["top2_logits_probs"][step]
         if tok == want:
             identical += 1
-        elif l1 - l2 <= NEAR_TIE and tok in fx["top2_ids"][step]:
+        elif l1 - l2 <= NEAR_TIE[name] and tok in fx["top2_ids"][step]:
             near_ties.append("step %d: device %d, oracle %d; oracle top-2 logits %.5f / %.5f" % (step, tok, want, l1, l2))
         else:
             failures.append("step %d: device %d, oracle %d (top-2 ids %s); oracle top-2 logits %.5f / %.5f"
@@ -187,7 +195,7 @@ def greedy_case(G, name):
     gc.close()
     gm.close()
     print("%s: %d of %d steps identical; near-tie steps: %s" % (name, identical, len(fx["tokens"]), near_ties or "none"))
-    n_close = sum(1 for t in fx["top2_logits_probs"] if t[0] - t[1] <= NEAR_TIE)
+    n_close = sum(1 for t in fx["top2_logits_probs"] if t[0] - t[1] <= NEAR_TIE[name])
     return identical, len(fx["tokens"]), near_ties, failures, n_close
 
 
@@ -204,4 +212,56 @@ def test_greedy_tokens_llama30b_u8(gpu):
     identical, total, near_ties, failures, n_close = greedy_case(gpu, "llama30b_u8_seed0_greedy.json")
     assert not failures, "\n".join(failures)
     assert identical + len(near_ties) == total and len(near_ties) <= n_close
-    assert identical >= total - 4
+    assert identical >= total - 8
+
+
+def test_u8_and_f16_kernels_agree_at_30b_depth(gpu):
+    """The uint8 kernels against the fp16 kernels on the same weight values (the uint8 model's
+    weights dequantised into an fp16 model), LLaMA-30B shape, teacher-forced on the fixture's tokens.
+    Both paths are held to the fixture's logits within the tolerance, and their mutual deviation
+    documents the noise floor that NEAR_TIE for this depth is taken from."""
+    G = gpu
+    path = os.path.join(GOLDEN, "llama30b_u8_seed0_greedy.json")
+    if not os.path.exists(path):
+        pytest.skip("fixture not generated")
+    fx = json.load(open(path))
+    kw = dict(dim=fx["dim"], multiple_of=fx["multiple_of"], n_heads=fx["n_heads"], n_layers=fx["n_layers"],
+              n_vocab=fx["n_vocab"], norm_eps=fx["norm_eps"], qblock=fx["qblock"], seed=fx["seed"],
+              weight_std=fx["weight_std"])
+    mu = G.P.Model(q_type=1, **kw)
+    mf = G.P.Model(q_type=0, **kw)
+    dim, ffn, vocab = fx["dim"], mu.ffn, fx["n_vocab"]
+    shapes = {1: (vocab, dim), 2: (vocab, dim)}
+    for l in range(fx["n_layers"]):
+        b = 16 + 16 * l
+        shapes.update({b: (dim, dim), b + 1: (dim, dim), b + 2: (dim, dim), b + 3: (dim, dim), b + 4: (ffn, dim),
+                       b + 5: (dim, ffn), b + 6: (ffn, dim)})
+    for sid, (rows, cols) in shapes.items():
+        codes, scales = mu.tensor_ptr(sid)
+        values, _ = mf.tensor_ptr(sid)
+        G.B.check(G.L().lcu_dequantize_absmax_u8(values, scales, codes, rows, cols, fx["qblock"], None))
+    G.L().lcu_sync(None)
+    cu = G.P.Context(mu, context_len=fx["context_len"], temperature=fx["temperature"])
+    cf = G.P.Context(mf, context_len=fx["context_len"], temperature=fx["temperature"])
+    feed = np.array(fx["prompt"], dtype=np.int16)
+    mutual, to_oracle = [], []
+    DEPTH_TOL = 2 * TOL  # TOL is the per-operator bar; sixty layers compound (largest seen: 1.1e-2)
+    for step, want in enumerate(fx["tokens"][:24]):
+        cu.next_token(feed)
+        cf.next_token(feed)
+        lu = cu.logits().astype(np.float32).ravel()
+        lf = cf.logits().astype(np.float32).ravel()
+        scale = np.abs(lf).max()
+        assert np.abs(lu - lf).max() / scale <= DEPTH_TOL
+        mutual.append(np.abs(lu - lf).mean())
+        l1, l2, _, _ = fx["top2_logits_probs"][step]
+        i1, i2 = fx["top2_ids"][step]
+        for dev in (lu, lf):
+            assert abs(dev[i1] - l1) / scale <= DEPTH_TOL and abs(dev[i2] - l2) / scale <= DEPTH_TOL
+            to_oracle += [abs(dev[i1] - l1), abs(dev[i2] - l2)]
+        feed = np.array([want], dtype=np.int16)
+    print("30B depth: mean |u8 - f16 kernels| %.4f, mean |device - oracle| at the top two %.4f"
+          % (np.mean(mutual), np.mean(to_oracle)))
+    assert np.mean(mutual) < 0.03 and np.mean(to_oracle) < 0.04
+    for o in (cu, cf, mu, mf):
+        o.close()

@@ -18,6 +18,7 @@ extern "C" {
 
 typedef struct lcu_model lcu_model;
 typedef struct lcu_context lcu_context;
+typedef struct lcu_vocab lcu_vocab;
 
 /* llama_params (llama_cu.h:280-291) from its fields; q_type 0 = fp16, 1 = uint8 */
 /* llama_model::create_synthetic (no reference counterpart: seeded random weights, norms = 1) */
@@ -29,6 +30,9 @@ lcu_model* lcu_model_create_synthetic(uint32_t dim, uint32_t multiple_of, uint32
 lcu_model* lcu_model_load(const char* model_dir, int context_len);
 void lcu_model_destroy(lcu_model*);
 uint32_t lcu_model_ffn_dim(const lcu_model*);                      /* llama_params::ffn_dim */
+/* the model's llama_params fields (llama_cu.h:280-291); q_type 0 = fp16, 1 = uint8 */
+void lcu_model_describe(const lcu_model*, uint32_t* dim, uint32_t* multiple_of, uint32_t* n_heads, uint32_t* n_layers,
+                        uint32_t* n_vocab, float* norm_eps, int* q_type, int* quantization_block_size);
 /* copies a weight matrix back to the host: stream id 1 tok_embeddings, 2 output, 16+16l+{0..6}
  * wq wk wv wo w1 w2 w3; `scales` may be NULL for fp16 models */
 int lcu_model_read_tensor(const lcu_model*, uint64_t stream_id, void* values, void* scales);
@@ -55,6 +59,20 @@ int lcu_context_read_hidden(lcu_context*, uint16_t* out, int rows);
 int lcu_context_read_kv(lcu_context*, int layer, uint16_t* k_out, uint16_t* v_out, int T);
 /* the hipStream_t (as void*) the context launches on, for event timing */
 void* lcu_context_stream(lcu_context*);
+
+/* mapped_buffer(path) + llama_vocabulary(buffer) (main.cpp:25,35; llama_cu.cu:1312-1339).  The
+ * file is checked first (entry table and piece offsets inside the file, pieces NUL-terminated):
+ * NULL if it cannot be read or is malformed, where the reference would read out of bounds. */
+lcu_vocab* lcu_vocab_load(const char* vocab_path);
+void lcu_vocab_destroy(lcu_vocab*);
+int lcu_vocab_size(const lcu_vocab*);                                /* tokens.size() */
+/* llama_vocabulary::tokenize(text, bos) (llama_cu.cu:1341-1360): writes at most `capacity` ids and
+ * returns how many the text has */
+int lcu_vocab_tokenize(lcu_vocab*, const char* text, size_t text_len, int bos, int16_t* out, int capacity);
+/* tokens[id].text (bytes, may contain NUL for the byte tokens 3..258) and .score; NULL / 0 if id is
+ * out of range */
+const char* lcu_vocab_piece(const lcu_vocab*, int id, size_t* len);
+float lcu_vocab_score(const lcu_vocab*, int id);
 
 #ifdef __cplusplus
 }

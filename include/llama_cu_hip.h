@@ -160,6 +160,12 @@ int lcu_fill_normal_f16(void* out_dev, size_t n, uint64_t seed, uint64_t stream_
                         void* stream);
 int lcu_fill_f16(void* out_dev, size_t n, uint16_t bits, void* stream);
 
+/* error_stats, transform.cu:99-150 (launch site 175): out3 = {mean squared difference, largest
+ * absolute difference, mean absolute difference} of two fp16 arrays of n elements, as fp32.
+ * Deterministic (partials are added in index order, where the reference uses atomics).  Uses the
+ * per-device workspace: calls that overlap on one device race. */
+int lcu_error_stats(void* out3_dev, const void* a_dev, const void* b_dev, size_t n, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -69,11 +69,13 @@ SIGNATURES = {
     "lcu_decode_logits": (i32, [vp, vp, vp, vp, vp, i32, i32, i32, f32, vp]),
     "lcu_fill_normal_f16": (i32, [vp, sz, u64, u64, f32, vp]),
     "lcu_fill_f16": (i32, [vp, sz, u16, vp]),
+    "lcu_error_stats": (i32, [vp, vp, vp, sz, vp]),
     # llama_cu_c.h
     "lcu_model_create_synthetic": (vp, [u32, u32, u32, u32, u32, f32, i32, i32, u64, f32]),
     "lcu_model_load": (vp, [C.c_char_p, i32]),
     "lcu_model_destroy": (None, [vp]),
     "lcu_model_ffn_dim": (u32, [vp]),
+    "lcu_model_describe": (None, [vp] + [C.POINTER(u32)] * 5 + [C.POINTER(f32), C.POINTER(i32), C.POINTER(i32)]),
     "lcu_model_read_tensor": (i32, [vp, u64, vp, vp]),
     "lcu_model_tensor_ptr": (i32, [vp, u64, C.POINTER(vp), C.POINTER(vp)]),
     "lcu_model_norm_ptr": (vp, [vp, i32]),
@@ -88,6 +90,12 @@ SIGNATURES = {
     "lcu_context_read_hidden": (i32, [vp, vp, i32]),
     "lcu_context_read_kv": (i32, [vp, i32, vp, vp, i32]),
     "lcu_context_stream": (vp, [vp]),
+    "lcu_vocab_load": (vp, [C.c_char_p]),
+    "lcu_vocab_destroy": (None, [vp]),
+    "lcu_vocab_size": (i32, [vp]),
+    "lcu_vocab_tokenize": (i32, [vp, C.c_char_p, sz, i32, vp, i32]),
+    "lcu_vocab_piece": (vp, [vp, i32, C.POINTER(sz)]),
+    "lcu_vocab_score": (f32, [vp, i32]),
 }
 
 
@@ -181,8 +189,12 @@ class Model:
                                                   qblock, seed, weight_std)
         if not self.h:
             raise LcuError("model creation failed: %s" % L.lcu_last_error().decode())
-        self.dim, self.n_heads, self.n_layers, self.n_vocab = dim, n_heads, n_layers, n_vocab
-        self.q_type, self.qblock = q_type, qblock
+        d, m, h, l, v = u32(), u32(), u32(), u32(), u32()
+        eps, qt, qb = f32(), i32(), i32()
+        L.lcu_model_describe(self.h, C.byref(d), C.byref(m), C.byref(h), C.byref(l), C.byref(v), C.byref(eps),
+                             C.byref(qt), C.byref(qb))
+        self.dim, self.multiple_of, self.n_heads, self.n_layers, self.n_vocab = d.value, m.value, h.value, l.value, v.value
+        self.norm_eps, self.q_type, self.qblock = eps.value, qt.value, (qb.value or qblock)
         self.ffn = L.lcu_model_ffn_dim(self.h)
 
     def tensor(self, stream_id, rows, cols):
@@ -271,6 +283,48 @@ class Context:
     def close(self):
         if getattr(self, "h", None):
             lib().lcu_context_destroy(self.h)
+            self.h = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+class Vocabulary:
+    """llama_vocabulary over a vocab file in the reference's format (host only, no GPU needed)."""
+
+    def __init__(self, path):
+        self.h = lib().lcu_vocab_load(path.encode())
+        if not self.h:
+            raise LcuError("could not load vocab file %s" % path)
+
+    def __len__(self):
+        return lib().lcu_vocab_size(self.h)
+
+    def tokenize(self, text, bos=True):
+        data = text.encode("utf-8") if isinstance(text, str) else bytes(text)
+        cap = 2 * len(data) + 8
+        out = (C.c_int16 * cap)()
+        n = lib().lcu_vocab_tokenize(self.h, data, len(data), 1 if bos else 0, out, cap)
+        if n < 0 or n > cap:
+            raise LcuError("lcu_vocab_tokenize returned %d" % n)
+        return list(out[:n])
+
+    def piece(self, token_id):
+        n = sz()
+        ptr = lib().lcu_vocab_piece(self.h, token_id, C.byref(n))
+        if not ptr:
+            raise IndexError(token_id)
+        return C.string_at(ptr, n.value)
+
+    def score(self, token_id):
+        return lib().lcu_vocab_score(self.h, token_id)
+
+    def close(self):
+        if getattr(self, "h", None):
+            lib().lcu_vocab_destroy(self.h)
             self.h = None
 
     def __del__(self):

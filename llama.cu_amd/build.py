@@ -9,6 +9,9 @@ LIB = os.path.join(PKG, "libllama_cu_amd.so")
 
 HIP_SOURCES = ["csrc/runtime.hip", "csrc/elementwise.hip", "csrc/gemv.hip", "csrc/gemm.hip", "csrc/attention.hip"]
 HOST_SOURCES = ["host/buffers.cpp", "host/params.cpp", "host/model.cpp", "host/tokenizer.cpp", "host/capi.cpp"]
+# command line programs linked against the library (found at run time next to bin/ through $ORIGIN)
+APPS = {"transform": "apps/transform.cpp", "llama_cu": "apps/llama_cu.cpp"}
+BIN = os.path.join(PKG, "bin")
 
 COMMON = ["-O3", "-std=c++17", "-fPIC", "-I" + os.path.join(ROOT, "include"), "-I" + os.path.join(PKG, "csrc"),
           "-I" + os.path.join(PKG, "host"), "-Wall", "-Wno-unused-function"]
@@ -41,6 +44,13 @@ def build(verbose=False):
         raise RuntimeError("hipcc failed")
     cmd = ["hipcc", "--offload-arch=gfx950", "-shared", "-o", LIB] + objs
     subprocess.check_call(cmd)
+    os.makedirs(BIN, exist_ok=True)
+    for name, src in APPS.items():
+        cmd = ["hipcc"] + COMMON + ["-x", "c++", os.path.join(PKG, src), "-o", os.path.join(BIN, name),
+               "-L" + PKG, "-lllama_cu_amd", "-Wl,-rpath,$ORIGIN/.."]
+        if verbose:
+            print(" ".join(cmd))
+        subprocess.check_call(cmd)
     return LIB
 
 

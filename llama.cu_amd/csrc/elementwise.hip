@@ -356,6 +356,55 @@ inline int grid_for(size_t n, int threads, int cap = 1 << 16) {
   return (int)(g < 1 ? 1 : (g > (size_t)cap ? cap : g));
 }
 
+
+// ---- error_stats, transform.cu:99-150: mean squared, largest absolute and mean absolute
+// difference of two fp16 arrays.  The reference adds its blocks' contributions with atomics, in
+// whatever order they arrive; here each workgroup writes its three partials and the last stage
+// adds them in index order, so the result is the same on every run.
+constexpr int ERR_BLOCKS = 256;
+
+__global__ __launch_bounds__(256) void error_stats_partial_kernel(float* __restrict__ partials,
+                                                                  const half_t* __restrict__ a,
+                                                                  const half_t* __restrict__ b, size_t n) {
+  __shared__ float red[3][4];
+  float sum_sq = 0.0f, mx = 0.0f, sum = 0.0f;
+  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (size_t)ERR_BLOCKS * 256) {
+    const float d = (float)a[i] - (float)b[i];
+    sum_sq = fmaf(d, d, sum_sq);
+    mx = fmaxf(mx, fabsf(d));
+    sum += fabsf(d);
+  }
+  sum_sq = wave_sum(sum_sq);
+  sum = wave_sum(sum);
+  mx = wave_max(mx);
+  if ((threadIdx.x & 63) == 0) {
+    red[0][threadIdx.x >> 6] = sum_sq;
+    red[1][threadIdx.x >> 6] = mx;
+    red[2][threadIdx.x >> 6] = sum;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    partials[blockIdx.x * 3 + 0] = (red[0][0] + red[0][1]) + (red[0][2] + red[0][3]);
+    partials[blockIdx.x * 3 + 1] = fmaxf(fmaxf(red[1][0], red[1][1]), fmaxf(red[1][2], red[1][3]));
+    partials[blockIdx.x * 3 + 2] = (red[2][0] + red[2][1]) + (red[2][2] + red[2][3]);
+  }
+}
+
+__global__ __launch_bounds__(64) void error_stats_final_kernel(float* __restrict__ out,
+                                                               const float* __restrict__ partials, size_t n) {
+  if (threadIdx.x != 0) return;
+  double sum_sq = 0.0, sum = 0.0;
+  float mx = 0.0f;
+  for (int i = 0; i < ERR_BLOCKS; ++i) {
+    sum_sq += (double)partials[i * 3 + 0];
+    mx = fmaxf(mx, partials[i * 3 + 1]);
+    sum += (double)partials[i * 3 + 2];
+  }
+  out[0] = (float)(sum_sq / (double)n);
+  out[1] = mx;
+  out[2] = (float)(sum / (double)n);
+}
+
 }  // namespace
 
 extern "C" {
@@ -532,6 +581,19 @@ int lcu_fill_f16(void* out_dev, size_t n, uint16_t bits, void* stream) {
   LCU_REQUIRE(out_dev || n == 0, "lcu_fill_f16: null pointer");
   if (n == 0) return LCU_OK;
   fill_u16_kernel<<<grid_for(n, 256, 4096), 256, 0, as_stream(stream)>>>((uint16_t*)out_dev, n, bits);
+  LCU_LAUNCH_CHECK();
+  return LCU_OK;
+}
+
+int lcu_error_stats(void* out3_dev, const void* a_dev, const void* b_dev, size_t n, void* stream) {
+  LCU_REQUIRE(out3_dev && a_dev && b_dev && n > 0, "lcu_error_stats: bad arguments");
+  device_state* st = current_device_state();
+  if (!st || !st->ready) return set_error(LCU_E_NOINIT, "lcu_error_stats: lcu_init has not run on this device");
+  float* partials = (float*)st->workspace;  // 256 x 3 floats of the per-device workspace
+  error_stats_partial_kernel<<<ERR_BLOCKS, 256, 0, as_stream(stream)>>>(partials, (const half_t*)a_dev,
+                                                                        (const half_t*)b_dev, n);
+  LCU_LAUNCH_CHECK();
+  error_stats_final_kernel<<<1, 64, 0, as_stream(stream)>>>((float*)out3_dev, partials, n);
   LCU_LAUNCH_CHECK();
   return LCU_OK;
 }

@@ -49,8 +49,8 @@ int lcu_init(int device) {
                      device, prop.gcnArchName);
   }
   st.compute_units = prop.multiProcessorCount;
-  // attention workspace: partial outputs of up to 64 heads x 32 splits x (128 + 2) floats,
-  // followed by one arrival counter per head
+  // per-device workspace for operators that reduce in two launches (lcu_error_stats: 256 x 3
+  // partial sums); calls that use it and overlap on one device race
   st.workspace_bytes = 4u << 20;
   LCU_HIP(hipMalloc(&st.workspace, st.workspace_bytes));
   LCU_HIP(hipMemset(st.workspace, 0, st.workspace_bytes));

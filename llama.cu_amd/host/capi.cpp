@@ -1,7 +1,9 @@
 // C handles over the C++ host interface; see llama_cu_c.h.
 #include "llama_cu_c.h"
 
+#include <cstring>
 #include <memory>
+#include <string>
 
 #include "model_impl.hpp"
 
@@ -16,6 +18,32 @@ struct lcu_context {
   std::unique_ptr<llama_context> context;
   llama_context_impl* impl() const { return static_cast<llama_context_impl*>(context.get()); }
 };
+
+struct lcu_vocab {
+  mapped_buffer file;
+  std::unique_ptr<llama_vocabulary> vocab;
+};
+
+namespace {
+// uint32 count, count x {uint32 offset, float score}, NUL-terminated pieces at the offsets
+bool vocab_file_is_sound(mapped_buffer const& f) {
+  if (!f.is_ok() || f.size() < sizeof(uint32_t)) return false;
+  const char* base = static_cast<const char*>(f.data());
+  uint32_t count;
+  memcpy(&count, base, sizeof(count));
+  const size_t table_end = sizeof(uint32_t) + (size_t)count * 8;
+  if (count > 32767 || table_end > f.size()) return false;
+  if (count == 0) return true;
+  if (base[f.size() - 1] != '\0') return false;  // every piece ends inside the file
+  for (uint32_t i = 0; i < count; ++i) {
+    uint32_t offset;
+    memcpy(&offset, base + sizeof(uint32_t) + (size_t)i * 8, sizeof(offset));
+    const bool by_text = i < 3 || i >= 259;  // ids 3..258 are bytes, their offsets are not read
+    if (by_text && (offset < table_end || offset >= f.size())) return false;
+  }
+  return true;
+}
+}  // namespace
 
 extern "C" {
 
@@ -74,6 +102,20 @@ lcu_model* lcu_model_load(const char* model_dir, int context_len) {
 void lcu_model_destroy(lcu_model* m) { delete m; }
 
 uint32_t lcu_model_ffn_dim(const lcu_model* m) { return m->model->params.ffn_dim(); }
+
+void lcu_model_describe(const lcu_model* m, uint32_t* dim, uint32_t* multiple_of, uint32_t* n_heads,
+                        uint32_t* n_layers, uint32_t* n_vocab, float* norm_eps, int* q_type,
+                        int* quantization_block_size) {
+  llama_params const& p = m->model->params;
+  if (dim) *dim = p.dim;
+  if (multiple_of) *multiple_of = p.multiple_of;
+  if (n_heads) *n_heads = p.n_heads;
+  if (n_layers) *n_layers = p.n_layers;
+  if (n_vocab) *n_vocab = p.n_vocab;
+  if (norm_eps) *norm_eps = p.norm_eps;
+  if (q_type) *q_type = p.q_type == quantization_type::uint8 ? 1 : 0;
+  if (quantization_block_size) *quantization_block_size = p.quantization_block_size;
+}
 
 int lcu_model_read_tensor(const lcu_model* m, uint64_t stream_id, void* values, void* scales) {
   weight_tensor const* t = m->impl()->tensor_by_stream(stream_id);
@@ -167,5 +209,42 @@ int lcu_context_read_kv(lcu_context* c, int layer, uint16_t* k_out, uint16_t* v_
 }
 
 void* lcu_context_stream(lcu_context* c) { return c->impl()->stream(); }
+
+lcu_vocab* lcu_vocab_load(const char* vocab_path) {
+  if (!vocab_path) return nullptr;
+  mapped_buffer file{std::string(vocab_path)};
+  if (!vocab_file_is_sound(file)) {
+    fprintf(stderr, "Could not load vocab file\n");
+    return nullptr;
+  }
+  auto* v = new lcu_vocab{std::move(file), nullptr};
+  v->vocab = std::make_unique<llama_vocabulary>(v->file);
+  return v;
+}
+
+void lcu_vocab_destroy(lcu_vocab* v) { delete v; }
+
+int lcu_vocab_size(const lcu_vocab* v) { return v ? (int)v->vocab->tokens.size() : 0; }
+
+int lcu_vocab_tokenize(lcu_vocab* v, const char* text, size_t text_len, int bos, int16_t* out, int capacity) {
+  if (!v || (!text && text_len) || (!out && capacity > 0)) return -1;
+  const std::vector<short> ids = v->vocab->tokenize(std::string_view(text ? text : "", text_len), bos != 0);
+  for (int i = 0; i < capacity && i < (int)ids.size(); ++i) out[i] = ids[i];
+  return (int)ids.size();
+}
+
+const char* lcu_vocab_piece(const lcu_vocab* v, int id, size_t* len) {
+  if (!v || id < 0 || id >= (int)v->vocab->tokens.size()) {
+    if (len) *len = 0;
+    return nullptr;
+  }
+  if (len) *len = v->vocab->tokens[id].text.size();
+  return v->vocab->tokens[id].text.data();
+}
+
+float lcu_vocab_score(const lcu_vocab* v, int id) {
+  if (!v || id < 0 || id >= (int)v->vocab->tokens.size()) return 0.0f;
+  return v->vocab->tokens[id].score;
+}
 
 }  // extern "C"

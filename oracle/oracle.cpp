@@ -425,6 +425,20 @@ void orc_embed_u8(uint16_t* out, const int16_t* ids, int n_ids, int dim, const u
   }
 }
 
+void orc_error_stats(float* out3, const uint16_t* a, const uint16_t* b, size_t n) {
+  double sum_sq = 0.0, sum = 0.0;
+  float mx = 0.0f;
+  for (size_t i = 0; i < n; ++i) {
+    const float d = h2f(a[i]) - h2f(b[i]);  // transform.cu:119
+    sum_sq += (double)d * (double)d;
+    mx = fmaxf(mx, fabsf(d));
+    sum += fabsf(d);
+  }
+  out3[0] = (float)(sum_sq / (double)n);
+  out3[1] = mx;
+  out3[2] = (float)(sum / (double)n);
+}
+
 int orc_argmax_first(const uint16_t* probs, int n) {
   int best = 0;
   for (int i = 1; i < n; ++i) {

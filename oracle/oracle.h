@@ -15,6 +15,7 @@
  *   orc_rms_norm, orc_rotary, orc_softmax_rows, orc_silu_mul, orc_matmul_qk, orc_matmul_qkv,
  *   orc_embed[_u8], orc_argmax_first : pinned by closed forms and float64 restatements written
  *       independently in numpy (tests/test_oracle_ops.py).
+ *   orc_error_stats : pinned by closed forms (tests/test_oracle_ops.py).
  *   orc_context_next_token : pinned by an independent numpy float64 forward pass on a tiny model
  *       (tolerance) and by the prefill-then-decode == longer-prefill invariant.
  * The reference holds no golden vectors for any of these (it has no tests), and its CUDA sources
@@ -77,6 +78,12 @@ void orc_embed_u8(uint16_t* out, const int16_t* ids, int n_ids, int dim, const u
                   const uint16_t* scales, int block);
 /* llama_cu.cu:1205-1209: first maximum of fp16 values compared as float */
 int orc_argmax_first(const uint16_t* probs, int n);
+
+/* error_stats, transform.cu:99-150: out3 = {mean of d^2, max |d|, mean |d|}, d = a[i] - b[i] in
+ * fp32, sums carried in double (the reference adds fp32 partials with atomics in arrival order,
+ * so its own result is only defined to fp32 summation accuracy).  Pinned by closed forms:
+ * identical arrays -> 0, a constant offset -> {c^2, c, c}, one differing element. */
+void orc_error_stats(float* out3, const uint16_t* a, const uint16_t* b, size_t n);
 
 /* ---- whole model: llama_cu.cu:882-1210 with seeded random weights instead of files ---- */
 typedef struct orc_model orc_model;

@@ -41,6 +41,8 @@ def lib():
         L.orc_silu_mul.argtypes = [vp, vp, vp, sz]
         L.orc_embed.argtypes = [vp, vp, i, i, vp]
         L.orc_embed_u8.argtypes = [vp, vp, i, i, vp, vp, i]
+        L.orc_error_stats.argtypes = [vp, vp, vp, sz]
+        L.orc_error_stats.restype = None
         L.orc_argmax_first.argtypes = [vp, i]
         L.orc_argmax_first.restype = i
         L.orc_model_create.argtypes = [i, i, i, i, i, f, i, i, u64, f]
@@ -187,6 +189,13 @@ def embed_u8(ids, codes, scales, block):
     scales = _f16(scales)
     out = np.empty((len(ids), codes.shape[1]), dtype=np.float16)
     lib().orc_embed_u8(_p(out), _p(ids), len(ids), codes.shape[1], _p(codes), _p(scales), block)
+    return out
+
+
+def error_stats(a, b):
+    a, b = _f16(a), _f16(b)
+    out = np.empty(3, dtype=np.float32)
+    lib().orc_error_stats(_p(out), _p(a), _p(b), a.size)
     return out
 
 

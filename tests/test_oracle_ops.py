@@ -243,3 +243,26 @@ def test_argmax_first_wins():
     assert O.argmax_first(p) == 1
     assert O.argmax_first(np.array([0.0, -0.0], dtype=np.float16)) == 0
     assert O.argmax_first(np.array([1, 2, 3], dtype=np.float16)) == 2
+
+
+# ------------------------------------------------------------------ error_stats (transform.cu:99-150)
+def test_error_stats_closed_forms():
+    a = f16(RNG.normal(0, 1, 10000))
+    assert (O.error_stats(a, a) == 0).all()
+    # a constant offset that fp16 represents exactly: every difference is 0.5
+    b = f16(np.arange(1000) * 0.5)
+    c = f16(np.arange(1000) * 0.5 + 0.5)
+    assert np.allclose(O.error_stats(c, b), [0.25, 0.5, 0.5], rtol=0, atol=0)
+    # one differing element among n: mse = d^2 / n, max = d, mean abs = d / n
+    d = a.copy()
+    d[1234] = np.float16(float(a[1234]) + 2.0)
+    delta = abs(float(d[1234]) - float(a[1234]))
+    mse, mx, mean = O.error_stats(d, a)
+    assert mx == np.float32(delta)
+    assert np.isclose(mse, delta * delta / a.size, rtol=1e-6) and np.isclose(mean, delta / a.size, rtol=1e-6)
+    # against float64 numpy on random data; sign of the difference must not matter
+    e = f16(RNG.normal(0, 1, 10000))
+    diff = a.astype(np.float32) - e.astype(np.float32)
+    want = [np.mean(diff.astype(np.float64) ** 2), np.max(np.abs(diff)), np.mean(np.abs(diff.astype(np.float64)))]
+    assert np.allclose(O.error_stats(a, e), want, rtol=1e-6)
+    assert np.allclose(O.error_stats(e, a), want, rtol=1e-6)

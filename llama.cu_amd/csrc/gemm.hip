@@ -5,7 +5,8 @@
 // the natural operand order of v_mfma_f32_32x32x16_f16: every lane feeds 8 consecutive k of one
 // row of lhs (A) and of one row of W (B).
 //
-//   - 256 threads = 4 wavefronts in a 2x2 grid; block tile BM x BN, K step 64
+//   - 4 wavefronts in a 2x2 grid over the block tile BM x BN, K step 64; optionally a second
+//     such group in the same workgroup that takes the other half of a 128-wide K stage
 //   - global -> registers -> LDS with two LDS buffers and two register stages: while the matrix
 //     cores work on K step t, step t+1 waits in registers and step t+2 is being fetched; LDS rows
 //     are padded by 16 bytes so the 16-byte operand reads of 16 neighbouring lanes fall in
@@ -28,9 +29,7 @@ int gemv_u8(half_t* out, const half_t* x, const uint8_t* W, const half_t* S, int
 
 namespace {
 
-constexpr int BK = 64;
-constexpr int LDK = BK + 8;  // halves per LDS row
-constexpr int THREADS = 256;
+constexpr int BK = 64;        // K extent one group of four wavefronts multiplies per stage
 constexpr int NUM_XCD = 8;
 
 __device__ __forceinline__ half2_t dequant2(uint32_t spread, half2_t scale2x) {
@@ -39,21 +38,31 @@ __device__ __forceinline__ half2_t dequant2(uint32_t spread, half2_t scale2x) {
   return t * scale2x;                                                                 // one rounding
 }
 
-// KTAIL: K is not a multiple of BK, so the last K step is partly out of range and must be zeroed
+// KS: groups of four wavefronts per workgroup.  A stage holds KS * 64 of K; group g multiplies
+// columns g*64 .. g*64+63 of it into its own accumulators, and the groups' accumulators are added
+// through LDS at the end (group 0 + group 1, a fixed order).  With KS = 2 every SIMD holds two
+// wavefronts of the same tile, so one can wait for LDS while the other feeds the matrix core --
+// what a second resident workgroup does when the grid has one to give, which at M = 512 it has not.
+// KTAIL: K is not a multiple of the stage, so the last stage is partly out of range and is zeroed
 // (costs selects in the loop; every model shape takes the KTAIL = false instantiation).
-template <int BM, int BN, bool U8, bool KTAIL>
-__global__ __launch_bounds__(THREADS, 2) void gemm_kernel(half_t* __restrict__ out, const half_t* __restrict__ A,
-                                                          const void* __restrict__ Wv, const half_t* __restrict__ S,
-                                                          int M, int K, int N, int block, float beta, int tiles_m,
-                                                          int tiles_n) {
-  constexpr int TM = BM / 64;  // 32x32 MFMA tiles per wavefront along M
+template <int BM, int BN, bool U8, bool KTAIL, int KS>
+__global__ __launch_bounds__(256 * KS, KS == 1 ? 2 : 1) void gemm_kernel(
+    half_t* __restrict__ out, const half_t* __restrict__ A, const void* __restrict__ Wv, const half_t* __restrict__ S,
+    int M, int K, int N, int block, float beta, int tiles_m, int tiles_n) {
+  constexpr int THREADS = 256 * KS;
+  constexpr int BKS = BK * KS;   // K extent of a stage
+  constexpr int LDK = BKS + 8;   // halves per LDS row: 16 bytes of padding keep 16-byte reads of 16 lanes in distinct banks
+  constexpr int TM = BM / 64;    // 32x32 MFMA tiles per wavefront along M
   constexpr int TN = BN / 64;
-  constexpr int A_CHUNKS = BM * BK / 8 / THREADS;                  // 16-byte chunks per thread
-  constexpr int B_CHUNKS = U8 ? BN * BK / 16 / THREADS : BN * BK / 8 / THREADS;
-  static_assert(A_CHUNKS >= 1 && B_CHUNKS >= 1, "tile too small for 256 threads");
+  constexpr int A_ROW = BKS / 8;                  // 16-byte chunks per tile row of lhs
+  constexpr int B_ROW = U8 ? BKS / 16 : BKS / 8;  // 16-byte chunks per tile row of W
+  constexpr int A_CHUNKS = BM * A_ROW / THREADS;  // chunks per thread
+  constexpr int B_CHUNKS = BN * B_ROW / THREADS;
+  static_assert(A_CHUNKS >= 1 && B_CHUNKS >= 1, "tile too small for the workgroup");
 
-  __shared__ __attribute__((aligned(16))) half_t As[2][BM * LDK];
-  __shared__ __attribute__((aligned(16))) half_t Bs[2][BN * LDK];
+  extern __shared__ __attribute__((aligned(16))) unsigned char gemm_lds[];
+  half_t* As = reinterpret_cast<half_t*>(gemm_lds);  // [2][BM * LDK]
+  half_t* Bs = As + 2 * BM * LDK;                    // [2][BN * LDK]
 
   // XCD-aware tile order: hardware deals consecutive workgroups round-robin to the 8 XCDs, so
   // give each XCD one contiguous run of the M-fastest tile sequence.
@@ -67,7 +76,8 @@ __global__ __launch_bounds__(THREADS, 2) void gemm_kernel(half_t* __restrict__ o
 
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
-  const int wm = (wave & 1) * (BM / 2), wn = (wave >> 1) * (BN / 2);
+  const int group = wave >> 2, w4 = wave & 3;
+  const int wm = (w4 & 1) * (BM / 2), wn = (w4 >> 1) * (BN / 2);
   const int nblk = U8 ? K / block : 0;
 
   // Per-thread byte offsets of its chunks from the operand bases; they do not change over the K
@@ -79,26 +89,26 @@ __global__ __launch_bounds__(THREADS, 2) void gemm_kernel(half_t* __restrict__ o
 #pragma unroll
   for (int i = 0; i < A_CHUNKS; ++i) {
     const int c = tid + i * THREADS;
-    a_k[i] = (c & 7) * 8;
-    a_off[i] = ((uint32_t)min(m0 + (c >> 3), M - 1) * (uint32_t)K + a_k[i]) * 2u;
+    a_k[i] = (c % A_ROW) * 8;
+    a_off[i] = ((uint32_t)min(m0 + c / A_ROW, M - 1) * (uint32_t)K + a_k[i]) * 2u;
   }
 #pragma unroll
   for (int i = 0; i < B_CHUNKS; ++i) {
     const int c = tid + i * THREADS;
+    const uint32_t row = (uint32_t)min(n0 + c / B_ROW, N - 1);
     if constexpr (U8) {
-      const uint32_t row = (uint32_t)min(n0 + (c >> 2), N - 1);
-      b_k[i] = (c & 3) * 16;
+      b_k[i] = (c % B_ROW) * 16;
       b_off[i] = row * (uint32_t)K + b_k[i];
       s_off[i] = row * (uint32_t)nblk;
     } else {
-      b_k[i] = (c & 7) * 8;
-      b_off[i] = ((uint32_t)min(n0 + (c >> 3), N - 1) * (uint32_t)K + b_k[i]) * 2u;
+      b_k[i] = (c % B_ROW) * 8;
+      b_off[i] = (row * (uint32_t)K + b_k[i]) * 2u;
     }
   }
   const char* Ab = (const char*)A;
   const char* Wb = (const char*)Wv;
 
-  // one K step of both operands in registers, as loaded from global memory
+  // one stage of both operands in registers, as loaded from global memory
   struct stage_t {
     half8_t ra[A_CHUNKS];
     half8_t rb[U8 ? 1 : B_CHUNKS];
@@ -137,12 +147,14 @@ __global__ __launch_bounds__(THREADS, 2) void gemm_kernel(half_t* __restrict__ o
   };
 
   auto store_tile = [&](const stage_t& st, int buf) {
+    half_t* Ad = As + buf * BM * LDK;
+    half_t* Bd = Bs + buf * BN * LDK;
 #pragma unroll
     for (int i = 0; i < A_CHUNKS; ++i) {
       const int c = tid + i * THREADS;
       half8_t v = st.ra[i];
       if constexpr (KTAIL) v = (st.k0 + a_k[i] < K) ? v : (half8_t)(0.0f);
-      *reinterpret_cast<half8_t*>(&As[buf][(c >> 3) * LDK + (c & 7) * 8]) = v;
+      *reinterpret_cast<half8_t*>(&Ad[(c / A_ROW) * LDK + a_k[i]]) = v;
     }
     if constexpr (U8) {
 #pragma unroll
@@ -159,7 +171,7 @@ __global__ __launch_bounds__(THREADS, 2) void gemm_kernel(half_t* __restrict__ o
         }
         half8_t lo = {d[0].x, d[0].y, d[1].x, d[1].y, d[2].x, d[2].y, d[3].x, d[3].y};
         half8_t hi = {d[4].x, d[4].y, d[5].x, d[5].y, d[6].x, d[6].y, d[7].x, d[7].y};
-        half_t* dst = &Bs[buf][(c >> 2) * LDK + (c & 3) * 16];
+        half_t* dst = &Bd[(c / B_ROW) * LDK + b_k[i]];
         *reinterpret_cast<half8_t*>(dst) = lo;
         *reinterpret_cast<half8_t*>(dst + 8) = hi;
       }
@@ -169,7 +181,7 @@ __global__ __launch_bounds__(THREADS, 2) void gemm_kernel(half_t* __restrict__ o
         const int c = tid + i * THREADS;
         half8_t v = st.rb[i];
         if constexpr (KTAIL) v = (st.k0 + b_k[i] < K) ? v : (half8_t)(0.0f);
-        *reinterpret_cast<half8_t*>(&Bs[buf][(c >> 3) * LDK + (c & 7) * 8]) = v;
+        *reinterpret_cast<half8_t*>(&Bd[(c / B_ROW) * LDK + b_k[i]]) = v;
       }
     }
   };
@@ -183,50 +195,87 @@ __global__ __launch_bounds__(THREADS, 2) void gemm_kernel(half_t* __restrict__ o
     }
   }
 
-  const int frag_row = lane & 31, frag_k = (lane >> 5) * 8;
+  // Operand fragments are read one 16-wide K slice ahead of the matrix instructions that use
+  // them (left to itself the compiler reads a fragment and waits for it in front of every
+  // instruction, and the matrix core idles for the LDS latency each time).
+  const int frag_row = lane & 31, frag_k = group * BK + (lane >> 5) * 8;
   auto compute = [&](int buf) {
+    const half_t* Ad = As + buf * BM * LDK + (wm + frag_row) * LDK + frag_k;
+    const half_t* Bd = Bs + buf * BN * LDK + (wn + frag_row) * LDK + frag_k;
+    half8_t fa[2][TM], fb[2][TN];
+    auto read_frags = [&](int slot, int ks) {
 #pragma unroll
-    for (int ks = 0; ks < BK; ks += 16) {
-      half8_t fa[TM], fb[TN];
+      for (int i = 0; i < TM; ++i) fa[slot][i] = *reinterpret_cast<const half8_t*>(Ad + i * 32 * LDK + ks);
 #pragma unroll
-      for (int i = 0; i < TM; ++i) {
-        fa[i] = *reinterpret_cast<const half8_t*>(&As[buf][(wm + i * 32 + frag_row) * LDK + ks + frag_k]);
-      }
+      for (int j = 0; j < TN; ++j) fb[slot][j] = *reinterpret_cast<const half8_t*>(Bd + j * 32 * LDK + ks);
+    };
+    read_frags(0, 0);
 #pragma unroll
-      for (int j = 0; j < TN; ++j) {
-        fb[j] = *reinterpret_cast<const half8_t*>(&Bs[buf][(wn + j * 32 + frag_row) * LDK + ks + frag_k]);
-      }
+    for (int s = 0; s < BK / 16; ++s) {
+      if (s + 1 < BK / 16) read_frags((s + 1) & 1, (s + 1) * 16);
+      __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int i = 0; i < TM; ++i) {
 #pragma unroll
         for (int j = 0; j < TN; ++j) {
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[i], fb[j], acc[i][j], 0, 0, 0);
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[s & 1][i], fb[s & 1][j], acc[i][j], 0, 0, 0);
         }
       }
+      __builtin_amdgcn_sched_barrier(0);
     }
   };
 
-  // Pipeline: LDS buffer t%2 holds K step t; one register stage holds step t+1 (requested one
-  // iteration ago) and the other receives step t+2 while the matrix cores work on step t.
+  // Pipeline: LDS buffer t%2 holds stage t; one register stage holds stage t+1 (requested one
+  // iteration ago) and the other receives stage t+2 while the matrix cores work on stage t.
   // Two iterations per trip so that the two register stages keep fixed names.
   stage_t s0, s1;
-  const int nt = (K + BK - 1) / BK;
+  const int nt = (K + BKS - 1) / BKS;
   load_tile(s0, 0);
-  if (nt > 1) load_tile(s1, BK);
+  if (nt > 1) load_tile(s1, BKS);
   store_tile(s0, 0);
   __syncthreads();
   for (int t = 0; t < nt; t += 2) {
-    // step t in LDS 0, step t+1 in s1
-    if (t + 2 < nt) load_tile(s0, (t + 2) * BK);
+    // stage t in LDS 0, stage t+1 in s1
+    if (t + 2 < nt) load_tile(s0, (t + 2) * BKS);
     compute(0);
     if (t + 1 < nt) store_tile(s1, 1);
     __syncthreads();
     if (t + 1 >= nt) break;
-    // step t+1 in LDS 1, step t+2 in s0
-    if (t + 3 < nt) load_tile(s1, (t + 3) * BK);
+    // stage t+1 in LDS 1, stage t+2 in s0
+    if (t + 3 < nt) load_tile(s1, (t + 3) * BKS);
     compute(1);
     if (t + 2 < nt) store_tile(s0, 0);
     __syncthreads();
+  }
+
+  // the groups' partial sums meet in LDS (every wavefront is past its last LDS read: each compute
+  // above is followed by a barrier); element (tile, v) of lane l sits at ((w4, tile, v), l)
+  if constexpr (KS == 2) {
+    float* part = reinterpret_cast<float*>(gemm_lds);
+    if (group == 1) {
+#pragma unroll
+      for (int i = 0; i < TM; ++i) {
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+#pragma unroll
+          for (int v = 0; v < 16; ++v) {
+            part[(((w4 * TM + i) * TN + j) * 16 + v) * 64 + lane] = acc[i][j][v];
+          }
+        }
+      }
+    }
+    __syncthreads();
+    if (group == 1) return;
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+#pragma unroll
+      for (int j = 0; j < TN; ++j) {
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          acc[i][j][v] += part[(((w4 * TM + i) * TN + j) * 16 + v) * 64 + lane];
+        }
+      }
+    }
   }
 
   // epilogue, llama_cu.cu:208-215: fp16(acc + beta * old).  Accumulator register v of lane l is
@@ -252,30 +301,52 @@ __global__ __launch_bounds__(THREADS, 2) void gemm_kernel(half_t* __restrict__ o
   }
 }
 
-template <int BM, int BN, bool U8>
+template <int BM, int BN, int KS>
+constexpr size_t gemm_lds_bytes() {
+  return (size_t)2 * (BM + BN) * (BK * KS + 8) * sizeof(half_t);
+}
+
+template <int BM, int BN, bool U8, bool KTAIL, int KS>
+int launch_one(half_t* out, const half_t* A, const void* W, const half_t* S, int M, int K, int N, int block,
+               float beta, int tiles_m, int tiles_n, hipStream_t st) {
+  constexpr size_t lds = gemm_lds_bytes<BM, BN, KS>();
+  static_assert(lds >= (size_t)BM * BN * 4 / 2 || KS == 1, "LDS must hold one group's accumulators");
+  auto kernel = gemm_kernel<BM, BN, U8, KTAIL, KS>;
+  if constexpr (lds > 64 * 1024) {
+    static bool raised[16] = {};  // per device, once
+    int dev = 0;
+    LCU_HIP(hipGetDevice(&dev));
+    if (!raised[dev & 15]) {
+      LCU_HIP(hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+      raised[dev & 15] = true;
+    }
+  }
+  kernel<<<tiles_m * tiles_n, 256 * KS, lds, st>>>(out, A, W, S, M, K, N, block, beta, tiles_m, tiles_n);
+  LCU_LAUNCH_CHECK();
+  return LCU_OK;
+}
+
+template <int BM, int BN, bool U8, int KS>
 int launch_gemm(half_t* out, const half_t* A, const void* W, const half_t* S, int M, int K, int N, int block,
                 float beta, hipStream_t st) {
   const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
-  if (K % BK == 0) {
-    gemm_kernel<BM, BN, U8, false><<<tiles_m * tiles_n, THREADS, 0, st>>>(out, A, W, S, M, K, N, block, beta, tiles_m,
-                                                                          tiles_n);
-  } else {
-    gemm_kernel<BM, BN, U8, true><<<tiles_m * tiles_n, THREADS, 0, st>>>(out, A, W, S, M, K, N, block, beta, tiles_m,
-                                                                         tiles_n);
+  if (K % (BK * KS) == 0) {
+    return launch_one<BM, BN, U8, false, KS>(out, A, W, S, M, K, N, block, beta, tiles_m, tiles_n, st);
   }
-  LCU_LAUNCH_CHECK();
-  return LCU_OK;
+  return launch_one<BM, BN, U8, true, KS>(out, A, W, S, M, K, N, block, beta, tiles_m, tiles_n, st);
 }
 
 template <bool U8>
 int dispatch_gemm(half_t* out, const half_t* A, const void* W, const half_t* S, int M, int K, int N, int block,
                   float beta, hipStream_t st) {
-  // 128x128 tiles when there are enough of them to give every compute unit one; else 128x64
+  // 128x128 tiles when there are enough of them to give every compute unit one (two fit a compute
+  // unit and desynchronise, which hides LDS latency better than the paired groups of KS = 2 do:
+  // 344 such tiles at N = 11008 beat 344 workgroups of eight wavefronts); else 128x64 tiles, of which there
+  // are then fewer than two per compute unit, so the workgroup brings the second group of
+  // wavefronts itself (M = 512, N = 4096: 35 us against 41 us, K = 11008: 100 us against 135 us).
   const long tiles128 = (long)((M + 127) / 128) * ((N + 127) / 128);
-  if (tiles128 >= 256) {
-    return launch_gemm<128, 128, U8>(out, A, W, S, M, K, N, block, beta, st);
-  }
-  return launch_gemm<128, 64, U8>(out, A, W, S, M, K, N, block, beta, st);
+  if (tiles128 >= 256) return launch_gemm<128, 128, U8, 1>(out, A, W, S, M, K, N, block, beta, st);
+  return launch_gemm<128, 64, U8, 2>(out, A, W, S, M, K, N, block, beta, st);
 }
 
 }  // namespace

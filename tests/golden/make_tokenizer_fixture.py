@@ -6,7 +6,7 @@ U+2581 replaced by a space), and SentencePiece's own encodings of the test strin
 
     python tests/golden/make_tokenizer_fixture.py
 
-Writes tests/golden/spm_bpe_vocab.bin and tests/golden/spm_bpe_cases.json.
+Writes tests/golden/spm_bpe.model, tests/golden/spm_bpe_vocab.bin and tests/golden/spm_bpe_cases.json.
 """
 import io
 import json
@@ -67,6 +67,8 @@ def main():
         character_coverage=1.0, normalization_rule_name="identity", add_dummy_prefix=True,
         remove_extra_whitespaces=False, split_digits=True, unk_id=0, bos_id=1, eos_id=2, pad_id=-1,
         num_threads=1, minloglevel=2)
+    with open(os.path.join(HERE, "spm_bpe.model"), "wb") as f:   # input of the vocabulary extractor's test
+        f.write(model.getvalue())
     sp = spm.SentencePieceProcessor(model_proto=model.getvalue())
     n = sp.vocab_size()
     pieces = [sp.id_to_piece(i).replace("▁", " ").encode("utf-8") for i in range(n)]

@@ -301,6 +301,231 @@ __global__ __launch_bounds__(256 * KS, KS == 1 ? 2 : 1) void gemm_kernel(
   }
 }
 
+// ---- fp16 weights, K a multiple of the stage: operands go from global memory straight into LDS
+// (global_load_lds_dwordx4: no staging registers, no LDS store instructions, and the wavefront
+// does not wait for a load before it can go on), through a ring of NS stages.
+//
+// A load instruction of one wavefront fills 1 KB of LDS, lane l at byte 16*l, so tile rows lie
+// densely (ROWB bytes each, no padding) and bank conflicts are avoided by permuting the 16-byte
+// chunks inside a row instead: the chunk that holds K offsets 8g..8g+7 of tile row r is stored at
+// chunk position g ^ f(r), f(r) = (r / RPB) % CR.  Sixteen lanes reading the same g from sixteen
+// consecutive rows then cover all 64 banks exactly once.
+//
+// Per iteration: wait until this wavefront's loads of stage t have landed, barrier (so everybody's
+// have), request stage t+NS-1 into the slot whose reads ended before that barrier, multiply
+// stage t.  The compiler does not track these loads against LDS reads; the waits are explicit.
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+
+template <int BM, int BN, int KS, int NS>
+__global__ __launch_bounds__(256 * KS, KS == 1 ? 2 : 1) void gemm_dl_kernel(
+    half_t* __restrict__ out, const half_t* __restrict__ A, const half_t* __restrict__ W, int M, int K, int N,
+    float beta, int tiles_m, int tiles_n) {
+  constexpr int NW = 4 * KS;                 // wavefronts
+  constexpr int BKS = BK * KS;               // K extent of a stage
+  constexpr int ROWB = BKS * 2;              // bytes of a tile row in LDS
+  constexpr int CR = ROWB / 16;              // 16-byte chunks per row: 8 or 16
+  constexpr int RPB = 16 / CR;               // tile rows per 256 bytes (one pass over the banks)
+  constexpr int PA = BM * CR / 64 / NW;      // load instructions per wavefront per stage, lhs
+  constexpr int PB = BN * CR / 64 / NW;      // and W
+  constexpr int A_BYTES = BM * ROWB;
+  constexpr int STAGE = (BM + BN) * ROWB;
+  constexpr int TM = BM / 64, TN = BN / 64;
+  static_assert(PA >= 1 && PB >= 1 && NS >= 2 && NS <= 4, "unsupported configuration");
+  static_assert((PA + PB) * (NS - 1) < 64, "vmcnt has 6 bits");
+
+  extern __shared__ __attribute__((aligned(16))) unsigned char gemm_lds[];
+
+  const int nb = tiles_m * tiles_n;
+  const int bid = blockIdx.x;
+  const int q = nb / NUM_XCD, r = nb % NUM_XCD;
+  const int xcd = bid % NUM_XCD, idx = bid / NUM_XCD;
+  const int logical = xcd * q + min(xcd, r) + idx;
+  const int tm = logical % tiles_m, tn = logical / tiles_m;
+  const int m0 = tm * BM, n0 = tn * BN;
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6;
+  const int group = wave >> 2, w4 = wave & 3;
+  const int wm = (w4 & 1) * (BM / 2), wn = (w4 >> 1) * (BN / 2);
+
+  // loader: instruction j of this wavefront fills LDS bytes [(wave + j*NW) * 1024, +1024) of the
+  // operand's region; lane l lands on tile row c / CR, chunk position c % CR, c = that index * 64 + l
+  uint32_t a_off[PA], b_off[PB];
+#pragma unroll
+  for (int j = 0; j < PA; ++j) {
+    const int c = (wave + j * NW) * 64 + lane;
+    const int row = c / CR, g = (c % CR) ^ ((row / RPB) % CR);
+    a_off[j] = ((uint32_t)min(m0 + row, M - 1) * (uint32_t)K + g * 8) * 2u;
+  }
+#pragma unroll
+  for (int j = 0; j < PB; ++j) {
+    const int c = (wave + j * NW) * 64 + lane;
+    const int row = c / CR, g = (c % CR) ^ ((row / RPB) % CR);
+    b_off[j] = ((uint32_t)min(n0 + row, N - 1) * (uint32_t)K + g * 8) * 2u;
+  }
+  const char* Ab = (const char*)A;
+  const char* Wb = (const char*)W;
+  using gptr = const __attribute__((address_space(1))) void*;
+  using lptr = __attribute__((address_space(3))) void*;
+  auto issue = [&](int stage, int slot) {
+    const size_t kb = (size_t)stage * (BKS * 2);
+    unsigned char* base = gemm_lds + slot * STAGE + wave * 1024;
+#pragma unroll
+    for (int j = 0; j < PA; ++j) {
+      __builtin_amdgcn_global_load_lds((gptr)(Ab + kb + a_off[j]), (lptr)(base + j * NW * 1024), 16, 0, 0);
+    }
+#pragma unroll
+    for (int j = 0; j < PB; ++j) {
+      __builtin_amdgcn_global_load_lds((gptr)(Wb + kb + b_off[j]), (lptr)(base + A_BYTES + j * NW * 1024), 16, 0, 0);
+    }
+  };
+
+  float16_t acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i) {
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      acc[i][j] = (float16_t)(0.0f);
+    }
+  }
+
+  // reader: chunk position of K slice s (16 wide) for this lane; the row term of f() is the same
+  // for every 32-row tile of the wavefront because 32 / RPB is a multiple of CR
+  const int frag_row = lane & 31;
+  const int fr = (frag_row / RPB) % CR;
+  const int gbase = group * 8 + (lane >> 5);
+  uint32_t pos[BK / 16];
+#pragma unroll
+  for (int s4 = 0; s4 < BK / 16; ++s4) pos[s4] = (uint32_t)(((gbase + 2 * s4) ^ fr) * 16);
+  const uint32_t a_row = (uint32_t)(wm + frag_row) * ROWB, b_row = (uint32_t)A_BYTES + (uint32_t)(wn + frag_row) * ROWB;
+
+  auto compute = [&](int slot) {
+    const unsigned char* base = gemm_lds + slot * STAGE;
+    half8_t fa[2][TM], fb[2][TN];
+    auto read_frags = [&](int buf, int s4) {
+#pragma unroll
+      for (int i = 0; i < TM; ++i) fa[buf][i] = *reinterpret_cast<const half8_t*>(base + a_row + i * 32 * ROWB + pos[s4]);
+#pragma unroll
+      for (int j = 0; j < TN; ++j) fb[buf][j] = *reinterpret_cast<const half8_t*>(base + b_row + j * 32 * ROWB + pos[s4]);
+    };
+    read_frags(0, 0);
+#pragma unroll
+    for (int s4 = 0; s4 < BK / 16; ++s4) {
+      if (s4 + 1 < BK / 16) read_frags((s4 + 1) & 1, s4 + 1);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int i = 0; i < TM; ++i) {
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[s4 & 1][i], fb[s4 & 1][j], acc[i][j], 0, 0, 0);
+        }
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+
+  const int nt = K / BKS;
+#pragma unroll
+  for (int s0 = 0; s0 < NS - 1; ++s0) {
+    if (s0 < nt) issue(s0, s0);
+  }
+  int slot = 0, fill = NS - 1;  // ring slots of stage t and of stage t + NS - 1
+  const int n_main = max(nt - (NS - 1), 0);
+  for (int t = 0; t < n_main; ++t) {
+    // stages t+1 .. t+NS-2 may stay in flight; stage t must have landed
+    wait_vmcnt<(NS - 2) * (PA + PB)>();
+    // a bare barrier: __syncthreads() would first wait for every outstanding load, the requests
+    // for the stages ahead included.  No LDS store is pending here (the loop has none) and the
+    // LDS reads of the previous stage were consumed by its matrix instructions.
+    asm volatile("s_barrier" ::: "memory");
+    issue(t + NS - 1, fill);
+    compute(slot);
+    slot = slot + 1 == NS ? 0 : slot + 1;
+    fill = fill + 1 == NS ? 0 : fill + 1;
+  }
+  // the last NS-1 stages: nothing left to request, so simply wait for everything
+  for (int t = n_main; t < nt; ++t) {
+    wait_vmcnt<0>();
+    asm volatile("s_barrier" ::: "memory");
+    compute(slot);
+    slot = slot + 1 == NS ? 0 : slot + 1;
+  }
+  __syncthreads();  // the last stage has been read by everybody: LDS is free for the partial sums
+
+  if constexpr (KS == 2) {
+    float* part = reinterpret_cast<float*>(gemm_lds);
+    if (group == 1) {
+#pragma unroll
+      for (int i = 0; i < TM; ++i) {
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+#pragma unroll
+          for (int v = 0; v < 16; ++v) {
+            part[(((w4 * TM + i) * TN + j) * 16 + v) * 64 + lane] = acc[i][j][v];
+          }
+        }
+      }
+    }
+    __syncthreads();
+    if (group == 1) return;
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+#pragma unroll
+      for (int j = 0; j < TN; ++j) {
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          acc[i][j][v] += part[(((w4 * TM + i) * TN + j) * 16 + v) * 64 + lane];
+        }
+      }
+    }
+  }
+
+  // epilogue as in gemm_kernel (llama_cu.cu:208-215)
+#pragma unroll
+  for (int i = 0; i < TM; ++i) {
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      const int gn = n0 + wn + j * 32 + (lane & 31);
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int gm = m0 + wm + i * 32 + (v >> 2) * 8 + (lane >> 5) * 4 + (v & 3);
+        if (gm < M && gn < N) {
+          half_t* p = out + (size_t)gm * N + gn;
+          float val = acc[i][j][v];
+          if (beta != 0.0f) {
+            val = fmaf(beta, (float)*p, val);
+          }
+          *p = round_f16(val);
+        }
+      }
+    }
+  }
+}
+
+template <int BM, int BN, int KS, int NS>
+int launch_dl(half_t* out, const half_t* A, const half_t* W, int M, int K, int N, float beta, hipStream_t st) {
+  constexpr size_t lds = (size_t)NS * (BM + BN) * (BK * KS * 2);
+  static_assert(lds <= 160 * 1024, "ring does not fit LDS");
+  static_assert(KS == 1 || lds >= (size_t)BM * BN * 4 / 2, "LDS must hold one group's accumulators");
+  const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
+  auto kernel = gemm_dl_kernel<BM, BN, KS, NS>;
+  if constexpr (lds > 64 * 1024) {
+    static bool raised[16] = {};  // per device, once
+    int dev = 0;
+    LCU_HIP(hipGetDevice(&dev));
+    if (!raised[dev & 15]) {
+      LCU_HIP(hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+      raised[dev & 15] = true;
+    }
+  }
+  kernel<<<tiles_m * tiles_n, 256 * KS, lds, st>>>(out, A, W, M, K, N, beta, tiles_m, tiles_n);
+  LCU_LAUNCH_CHECK();
+  return LCU_OK;
+}
+
 template <int BM, int BN, int KS>
 constexpr size_t gemm_lds_bytes() {
   return (size_t)2 * (BM + BN) * (BK * KS + 8) * sizeof(half_t);
@@ -345,6 +570,12 @@ int dispatch_gemm(half_t* out, const half_t* A, const void* W, const half_t* S, 
   // are then fewer than two per compute unit, so the workgroup brings the second group of
   // wavefronts itself (M = 512, N = 4096: 35 us against 41 us, K = 11008: 100 us against 135 us).
   const long tiles128 = (long)((M + 127) / 128) * ((N + 127) / 128);
+  if constexpr (!U8) {
+    if (K % 128 == 0) {  // fp16 weights, whole stages: the direct-to-LDS kernels
+      if (tiles128 >= 256) return launch_dl<128, 128, 1, 2>(out, A, (const half_t*)W, M, K, N, beta, st);
+      return launch_dl<128, 64, 2, 3>(out, A, (const half_t*)W, M, K, N, beta, st);
+    }
+  }
   if (tiles128 >= 256) return launch_gemm<128, 128, U8, 1>(out, A, W, S, M, K, N, block, beta, st);
   return launch_gemm<128, 64, U8, 2>(out, A, W, S, M, K, N, block, beta, st);
 }

@@ -17,6 +17,8 @@
 //   - block index -> tile mapping keeps the tiles that share a slice of W on one XCD (one L2)
 //   - no padding rows: rows >= M and columns >= N are masked instead of the reference's zeroed
 //     "gutter" (llama_cu.h:236-242)
+#include <type_traits>
+
 #include "common.hpp"
 
 using namespace lcu;
@@ -319,11 +321,20 @@ __device__ __forceinline__ void wait_vmcnt() {
   asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
 }
 
-template <int BM, int BN, int KS, int NS>
-__global__ __launch_bounds__(256 * KS, KS == 1 ? 2 : 1) void gemm_dl_kernel(
+// WM x WN wavefronts tile the block (each a (BM/WM) x (BN/WN) sub-tile of 32x32 matrix-instruction
+// tiles), times KS groups along K.
+//
+// PF > 0 adds one more wavefront that computes nothing: it touches one word of every 128-byte line
+// of the stage PF stages ahead of the loaders, so that the line is in L2 when they ask for it.
+// Without it a sixth of the requests (the first touch of each W line, and of each lhs line per
+// XCD) come from HBM with about 2.4 us of latency, every stage waits at its barrier for the
+// slowest of its loads, and LDS cannot hold enough stages in flight to cover that.
+template <int BM, int BN, int WM, int WN, int KS, int NS, int PF>
+__global__ __launch_bounds__(64 * (WM * WN * KS + (PF > 0 ? 1 : 0)), WM * WN * KS <= 4 ? 2 : 1) void gemm_dl_kernel(
     half_t* __restrict__ out, const half_t* __restrict__ A, const half_t* __restrict__ W, int M, int K, int N,
     float beta, int tiles_m, int tiles_n) {
-  constexpr int NW = 4 * KS;                 // wavefronts
+  constexpr int NG = WM * WN;                // wavefronts of one group
+  constexpr int NW = NG * KS;                // wavefronts
   constexpr int BKS = BK * KS;               // K extent of a stage
   constexpr int ROWB = BKS * 2;              // bytes of a tile row in LDS
   constexpr int CR = ROWB / 16;              // 16-byte chunks per row: 8 or 16
@@ -332,7 +343,7 @@ __global__ __launch_bounds__(256 * KS, KS == 1 ? 2 : 1) void gemm_dl_kernel(
   constexpr int PB = BN * CR / 64 / NW;      // and W
   constexpr int A_BYTES = BM * ROWB;
   constexpr int STAGE = (BM + BN) * ROWB;
-  constexpr int TM = BM / 64, TN = BN / 64;
+  constexpr int TM = BM / (32 * WM), TN = BN / (32 * WN);
   static_assert(PA >= 1 && PB >= 1 && NS >= 2 && NS <= 4, "unsupported configuration");
   static_assert((PA + PB) * (NS - 1) < 64, "vmcnt has 6 bits");
 
@@ -348,8 +359,8 @@ __global__ __launch_bounds__(256 * KS, KS == 1 ? 2 : 1) void gemm_dl_kernel(
 
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
-  const int group = wave >> 2, w4 = wave & 3;
-  const int wm = (w4 & 1) * (BM / 2), wn = (w4 >> 1) * (BN / 2);
+  const int group = wave / NG, w4 = wave % NG;
+  const int wm = (w4 % WM) * (BM / WM), wn = (w4 / WM) * (BN / WN);
 
   // loader: instruction j of this wavefront fills LDS bytes [(wave + j*NW) * 1024, +1024) of the
   // operand's region; lane l lands on tile row c / CR, chunk position c % CR, c = that index * 64 + l
@@ -370,17 +381,20 @@ __global__ __launch_bounds__(256 * KS, KS == 1 ? 2 : 1) void gemm_dl_kernel(
   const char* Wb = (const char*)W;
   using gptr = const __attribute__((address_space(1))) void*;
   using lptr = __attribute__((address_space(3))) void*;
-  auto issue = [&](int stage, int slot) {
+  // load instruction `idx` (0 .. PA+PB-1) of this wavefront for K stage `stage` into ring slot `slot`
+  auto issue_one = [&](int stage, int slot, int idx) {
     const size_t kb = (size_t)stage * (BKS * 2);
     unsigned char* base = gemm_lds + slot * STAGE + wave * 1024;
-#pragma unroll
-    for (int j = 0; j < PA; ++j) {
-      __builtin_amdgcn_global_load_lds((gptr)(Ab + kb + a_off[j]), (lptr)(base + j * NW * 1024), 16, 0, 0);
+    if (idx < PA) {
+      __builtin_amdgcn_global_load_lds((gptr)(Ab + kb + a_off[idx]), (lptr)(base + idx * NW * 1024), 16, 0, 0);
+    } else {
+      __builtin_amdgcn_global_load_lds((gptr)(Wb + kb + b_off[idx - PA]), (lptr)(base + A_BYTES + (idx - PA) * NW * 1024),
+                                       16, 0, 0);
     }
+  };
+  auto issue = [&](int stage, int slot) {
 #pragma unroll
-    for (int j = 0; j < PB; ++j) {
-      __builtin_amdgcn_global_load_lds((gptr)(Wb + kb + b_off[j]), (lptr)(base + A_BYTES + j * NW * 1024), 16, 0, 0);
-    }
+    for (int idx = 0; idx < PA + PB; ++idx) issue_one(stage, slot, idx);
   };
 
   float16_t acc[TM][TN];
@@ -402,7 +416,12 @@ __global__ __launch_bounds__(256 * KS, KS == 1 ? 2 : 1) void gemm_dl_kernel(
   for (int s4 = 0; s4 < BK / 16; ++s4) pos[s4] = (uint32_t)(((gbase + 2 * s4) ^ fr) * 16);
   const uint32_t a_row = (uint32_t)(wm + frag_row) * ROWB, b_row = (uint32_t)A_BYTES + (uint32_t)(wn + frag_row) * ROWB;
 
-  auto compute = [&](int slot) {
+  // Multiplies the stage in ring slot `slot`.  With FETCH, the loads of K stage `next` (into slot
+  // `fill`) are requested a few at a time between the K slices: a wavefront that requests all of
+  // them at once sits in the issue queue behind the other wavefronts' requests (the texture
+  // addresser takes 16 cycles per request) before it can start to multiply.
+  auto compute = [&](int slot, auto fetch, int next, int fill) {
+    constexpr bool FETCH = decltype(fetch)::value;
     const unsigned char* base = gemm_lds + slot * STAGE;
     half8_t fa[2][TM], fb[2][TN];
     auto read_frags = [&](int buf, int s4) {
@@ -412,9 +431,14 @@ __global__ __launch_bounds__(256 * KS, KS == 1 ? 2 : 1) void gemm_dl_kernel(
       for (int j = 0; j < TN; ++j) fb[buf][j] = *reinterpret_cast<const half8_t*>(base + b_row + j * 32 * ROWB + pos[s4]);
     };
     read_frags(0, 0);
+    constexpr int S4 = BK / 16, P = PA + PB;
 #pragma unroll
-    for (int s4 = 0; s4 < BK / 16; ++s4) {
-      if (s4 + 1 < BK / 16) read_frags((s4 + 1) & 1, s4 + 1);
+    for (int s4 = 0; s4 < S4; ++s4) {
+      if (s4 + 1 < S4) read_frags((s4 + 1) & 1, s4 + 1);
+      if constexpr (FETCH) {
+#pragma unroll
+        for (int idx = s4 * P / S4; idx < (s4 + 1) * P / S4; ++idx) issue_one(next, fill, idx);
+      }
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int i = 0; i < TM; ++i) {
@@ -428,6 +452,44 @@ __global__ __launch_bounds__(256 * KS, KS == 1 ? 2 : 1) void gemm_dl_kernel(
   };
 
   const int nt = K / BKS;
+  if constexpr (PF > 0) {
+    if (wave == NW) {
+      constexpr int LA = BM / 64, LB = BN / 64, LK = ROWB / 128;  // lines: 64 rows per instruction, LK per row and stage
+      uint32_t pa[LA], pb[LB];
+#pragma unroll
+      for (int i = 0; i < LA; ++i) pa[i] = (uint32_t)min(m0 + i * 64 + lane, M - 1) * (uint32_t)K * 2u;
+#pragma unroll
+      for (int i = 0; i < LB; ++i) pb[i] = (uint32_t)min(n0 + i * 64 + lane, N - 1) * (uint32_t)K * 2u;
+      uint32_t ring[PF][(LA + LB) * LK];
+      uint32_t sink = 0;
+      auto touch = [&](int d, int stage) {
+        const size_t kb = (size_t)min(stage, nt - 1) * (BKS * 2);
+#pragma unroll
+        for (int l = 0; l < LK; ++l) {
+#pragma unroll
+          for (int i = 0; i < LA; ++i) ring[d][(i * LK) + l] = *reinterpret_cast<const uint32_t*>(Ab + kb + l * 128 + pa[i]);
+#pragma unroll
+          for (int i = 0; i < LB; ++i) ring[d][(LA + i) * LK + l] = *reinterpret_cast<const uint32_t*>(Wb + kb + l * 128 + pb[i]);
+        }
+      };
+#pragma unroll
+      for (int d = 0; d < PF; ++d) touch(d, NS - 1 + d);
+      // one barrier per stage, as the other wavefronts execute
+      for (int t = 0; t < nt; t += PF) {
+#pragma unroll
+        for (int d = 0; d < PF; ++d) {
+          if (t + d < nt) {
+#pragma unroll
+            for (int i = 0; i < (LA + LB) * LK; ++i) sink ^= ring[d][i];  // waits for the oldest touch only
+            touch(d, NS - 1 + t + d + PF);
+            asm volatile("s_barrier" ::: "memory");
+          }
+        }
+      }
+      asm volatile("" ::"v"(sink));  // the touched words are used, so the loads stay
+      return;
+    }
+  }
 #pragma unroll
   for (int s0 = 0; s0 < NS - 1; ++s0) {
     if (s0 < nt) issue(s0, s0);
@@ -441,8 +503,7 @@ __global__ __launch_bounds__(256 * KS, KS == 1 ? 2 : 1) void gemm_dl_kernel(
     // for the stages ahead included.  No LDS store is pending here (the loop has none) and the
     // LDS reads of the previous stage were consumed by its matrix instructions.
     asm volatile("s_barrier" ::: "memory");
-    issue(t + NS - 1, fill);
-    compute(slot);
+    compute(slot, std::true_type{}, t + NS - 1, fill);
     slot = slot + 1 == NS ? 0 : slot + 1;
     fill = fill + 1 == NS ? 0 : fill + 1;
   }
@@ -450,7 +511,7 @@ __global__ __launch_bounds__(256 * KS, KS == 1 ? 2 : 1) void gemm_dl_kernel(
   for (int t = n_main; t < nt; ++t) {
     wait_vmcnt<0>();
     asm volatile("s_barrier" ::: "memory");
-    compute(slot);
+    compute(slot, std::false_type{}, 0, 0);
     slot = slot + 1 == NS ? 0 : slot + 1;
   }
   __syncthreads();  // the last stage has been read by everybody: LDS is free for the partial sums
@@ -505,13 +566,13 @@ __global__ __launch_bounds__(256 * KS, KS == 1 ? 2 : 1) void gemm_dl_kernel(
   }
 }
 
-template <int BM, int BN, int KS, int NS>
+template <int BM, int BN, int WM, int WN, int KS, int NS, int PF>
 int launch_dl(half_t* out, const half_t* A, const half_t* W, int M, int K, int N, float beta, hipStream_t st) {
   constexpr size_t lds = (size_t)NS * (BM + BN) * (BK * KS * 2);
   static_assert(lds <= 160 * 1024, "ring does not fit LDS");
   static_assert(KS == 1 || lds >= (size_t)BM * BN * 4 / 2, "LDS must hold one group's accumulators");
   const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
-  auto kernel = gemm_dl_kernel<BM, BN, KS, NS>;
+  auto kernel = gemm_dl_kernel<BM, BN, WM, WN, KS, NS, PF>;
   if constexpr (lds > 64 * 1024) {
     static bool raised[16] = {};  // per device, once
     int dev = 0;
@@ -521,7 +582,7 @@ int launch_dl(half_t* out, const half_t* A, const half_t* W, int M, int K, int N
       raised[dev & 15] = true;
     }
   }
-  kernel<<<tiles_m * tiles_n, 256 * KS, lds, st>>>(out, A, W, M, K, N, beta, tiles_m, tiles_n);
+  kernel<<<tiles_m * tiles_n, 64 * (WM * WN * KS + (PF > 0 ? 1 : 0)), lds, st>>>(out, A, W, M, K, N, beta, tiles_m, tiles_n);
   LCU_LAUNCH_CHECK();
   return LCU_OK;
 }
@@ -572,8 +633,10 @@ int dispatch_gemm(half_t* out, const half_t* A, const void* W, const half_t* S, 
   const long tiles128 = (long)((M + 127) / 128) * ((N + 127) / 128);
   if constexpr (!U8) {
     if (K % 128 == 0) {  // fp16 weights, whole stages: the direct-to-LDS kernels
-      if (tiles128 >= 256) return launch_dl<128, 128, 1, 2>(out, A, (const half_t*)W, M, K, N, beta, st);
-      return launch_dl<128, 64, 2, 3>(out, A, (const half_t*)W, M, K, N, beta, st);
+      const long tiles256 = (long)((M + 255) / 256) * ((N + 127) / 128);
+      if (tiles256 >= 160) return launch_dl<256, 128, 4, 2, 1, 3, 0>(out, A, (const half_t*)W, M, K, N, beta, st);
+      if (tiles128 >= 256) return launch_dl<128, 128, 2, 2, 1, 2, 0>(out, A, (const half_t*)W, M, K, N, beta, st);
+      return launch_dl<128, 64, 2, 2, 2, 3, 0>(out, A, (const half_t*)W, M, K, N, beta, st);
     }
   }
   if (tiles128 >= 256) return launch_gemm<128, 128, U8, 1>(out, A, W, S, M, K, N, block, beta, st);

@@ -324,13 +324,11 @@ __device__ __forceinline__ void wait_vmcnt() {
 // WM x WN wavefronts tile the block (each a (BM/WM) x (BN/WN) sub-tile of 32x32 matrix-instruction
 // tiles), times KS groups along K.
 //
-// PF > 0 adds one more wavefront that computes nothing: it touches one word of every 128-byte line
-// of the stage PF stages ahead of the loaders, so that the line is in L2 when they ask for it.
-// Without it a sixth of the requests (the first touch of each W line, and of each lhs line per
-// XCD) come from HBM with about 2.4 us of latency, every stage waits at its barrier for the
-// slowest of its loads, and LDS cannot hold enough stages in flight to cover that.
-template <int BM, int BN, int WM, int WN, int KS, int NS, int PF>
-__global__ __launch_bounds__(64 * (WM * WN * KS + (PF > 0 ? 1 : 0)), WM * WN * KS <= 4 ? 2 : 1) void gemm_dl_kernel(
+// Tried and dropped: an extra wavefront that touches the lines of a stage several stages ahead so
+// that the loaders hit L2.  About a sixth of the requests come from HBM, but the touches (64
+// separate lines per instruction) cost the texture addresser more than the misses cost the ring.
+template <int BM, int BN, int WM, int WN, int KS, int NS>
+__global__ __launch_bounds__(64 * WM * WN * KS, WM * WN * KS <= 4 ? 2 : 1) void gemm_dl_kernel(
     half_t* __restrict__ out, const half_t* __restrict__ A, const half_t* __restrict__ W, int M, int K, int N,
     float beta, int tiles_m, int tiles_n) {
   constexpr int NG = WM * WN;                // wavefronts of one group
@@ -416,103 +414,109 @@ __global__ __launch_bounds__(64 * (WM * WN * KS + (PF > 0 ? 1 : 0)), WM * WN * K
   for (int s4 = 0; s4 < BK / 16; ++s4) pos[s4] = (uint32_t)(((gbase + 2 * s4) ^ fr) * 16);
   const uint32_t a_row = (uint32_t)(wm + frag_row) * ROWB, b_row = (uint32_t)A_BYTES + (uint32_t)(wn + frag_row) * ROWB;
 
-  // Multiplies the stage in ring slot `slot`.  With FETCH, the loads of K stage `next` (into slot
-  // `fill`) are requested a few at a time between the K slices: a wavefront that requests all of
-  // them at once sits in the issue queue behind the other wavefronts' requests (the texture
-  // addresser takes 16 cycles per request) before it can start to multiply.
-  auto compute = [&](int slot, auto fetch, int next, int fill) {
-    constexpr bool FETCH = decltype(fetch)::value;
-    const unsigned char* base = gemm_lds + slot * STAGE;
-    half8_t fa[2][TM], fb[2][TN];
-    auto read_frags = [&](int buf, int s4) {
+  // ---- the stage loop, scheduled by hand ------------------------------------------------------
+  // The LDS reads and their waits are written as inline assembly: with global_load_lds requests
+  // outstanding the compiler waits for *every* LDS read in front of each matrix instruction group
+  // (it models the requests like FLAT accesses), which exposes the LDS latency four times per
+  // stage.  Here a group waits only for its own fragments (lgkmcnt counts LDS reads in order;
+  // the global_load_lds requests count in vmcnt), and the synchronisation for the next stage
+  // sits in front of the last group, so the first fragments of the next stage are already on
+  // their way while that group runs and the matrix core never drains at a stage boundary.
+  //
+  // K slice s of a stage uses fragment buffer s & 1.  Per stage and wavefront:
+  //   slices 0..2: read slice s+1 | wait for slice s | request a third of the stage NS-1 ahead | multiply s
+  //   slice 3:     wait for slice 3 (nothing else is pending: this wavefront is done reading the
+  //                stage) | wait for the own requests of the next stage | barrier | read slice 0 of
+  //                the next stage | multiply 3
+  constexpr int S4 = BK / 16, P = PA + PB;
+  static_assert(S4 == 4, "the schedule below is written for four K slices per stage");
+  const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char*)gemm_lds;
+  half8_t fa[2][TM], fb[2][TN];
+  auto read_frags = [&](int buf, int slot, int s4) {
+    const uint32_t pa = lds0 + slot * STAGE + a_row + pos[s4], pb = lds0 + slot * STAGE + b_row + pos[s4];
 #pragma unroll
-      for (int i = 0; i < TM; ++i) fa[buf][i] = *reinterpret_cast<const half8_t*>(base + a_row + i * 32 * ROWB + pos[s4]);
+    for (int i = 0; i < TM; ++i) {
+      asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(fa[buf][i]) : "v"(pa), "n"(i * 32 * ROWB));
+    }
 #pragma unroll
-      for (int j = 0; j < TN; ++j) fb[buf][j] = *reinterpret_cast<const half8_t*>(base + b_row + j * 32 * ROWB + pos[s4]);
-    };
-    read_frags(0, 0);
-    constexpr int S4 = BK / 16, P = PA + PB;
+    for (int j = 0; j < TN; ++j) {
+      asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(fb[buf][j]) : "v"(pb), "n"(j * 32 * ROWB));
+    }
+  };
+  // the fragments of `buf` become usable only after the wait: redefine them behind it
+  auto frags_ready = [&](int buf) {
 #pragma unroll
-    for (int s4 = 0; s4 < S4; ++s4) {
-      if (s4 + 1 < S4) read_frags((s4 + 1) & 1, s4 + 1);
+    for (int i = 0; i < TM; ++i) asm volatile("" : "+v"(fa[buf][i]));
+#pragma unroll
+    for (int j = 0; j < TN; ++j) asm volatile("" : "+v"(fb[buf][j]));
+  };
+  auto multiply = [&](int buf) {
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+#pragma unroll
+      for (int j = 0; j < TN; ++j) {
+        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[buf][i], fb[buf][j], acc[i][j], 0, 0, 0);
+      }
+    }
+  };
+  // one stage; FETCH: request stage `next` into slot `fill`; MORE: another stage follows (in
+  // `nslot`), whose own requests are complete once at most PEND requests are outstanding
+  auto stage = [&](int slot, auto fetch, int next, int fill, auto more, auto pend, int nslot) {
+    constexpr bool FETCH = decltype(fetch)::value, MORE = decltype(more)::value;
+    constexpr int PEND = decltype(pend)::value;
+#pragma unroll
+    for (int s4 = 0; s4 < 3; ++s4) {
+      read_frags((s4 + 1) & 1, slot, s4 + 1);
+      asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(TM + TN) : "memory");
+      frags_ready(s4 & 1);
       if constexpr (FETCH) {
 #pragma unroll
-        for (int idx = s4 * P / S4; idx < (s4 + 1) * P / S4; ++idx) issue_one(next, fill, idx);
+        for (int idx = s4 * P / 3; idx < (s4 + 1) * P / 3; ++idx) issue_one(next, fill, idx);
       }
-      __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-      for (int i = 0; i < TM; ++i) {
-#pragma unroll
-        for (int j = 0; j < TN; ++j) {
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[s4 & 1][i], fb[s4 & 1][j], acc[i][j], 0, 0, 0);
-        }
-      }
-      __builtin_amdgcn_sched_barrier(0);
+      multiply(s4 & 1);
     }
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    frags_ready(1);
+    if constexpr (MORE) {
+      wait_vmcnt<PEND>();
+      asm volatile("s_barrier" ::: "memory");
+      read_frags(0, nslot, 0);
+    }
+    multiply(1);
   };
 
   const int nt = K / BKS;
-  if constexpr (PF > 0) {
-    if (wave == NW) {
-      constexpr int LA = BM / 64, LB = BN / 64, LK = ROWB / 128;  // lines: 64 rows per instruction, LK per row and stage
-      uint32_t pa[LA], pb[LB];
-#pragma unroll
-      for (int i = 0; i < LA; ++i) pa[i] = (uint32_t)min(m0 + i * 64 + lane, M - 1) * (uint32_t)K * 2u;
-#pragma unroll
-      for (int i = 0; i < LB; ++i) pb[i] = (uint32_t)min(n0 + i * 64 + lane, N - 1) * (uint32_t)K * 2u;
-      uint32_t ring[PF][(LA + LB) * LK];
-      uint32_t sink = 0;
-      auto touch = [&](int d, int stage) {
-        const size_t kb = (size_t)min(stage, nt - 1) * (BKS * 2);
-#pragma unroll
-        for (int l = 0; l < LK; ++l) {
-#pragma unroll
-          for (int i = 0; i < LA; ++i) ring[d][(i * LK) + l] = *reinterpret_cast<const uint32_t*>(Ab + kb + l * 128 + pa[i]);
-#pragma unroll
-          for (int i = 0; i < LB; ++i) ring[d][(LA + i) * LK + l] = *reinterpret_cast<const uint32_t*>(Wb + kb + l * 128 + pb[i]);
-        }
-      };
-#pragma unroll
-      for (int d = 0; d < PF; ++d) touch(d, NS - 1 + d);
-      // one barrier per stage, as the other wavefronts execute
-      for (int t = 0; t < nt; t += PF) {
-#pragma unroll
-        for (int d = 0; d < PF; ++d) {
-          if (t + d < nt) {
-#pragma unroll
-            for (int i = 0; i < (LA + LB) * LK; ++i) sink ^= ring[d][i];  // waits for the oldest touch only
-            touch(d, NS - 1 + t + d + PF);
-            asm volatile("s_barrier" ::: "memory");
-          }
-        }
-      }
-      asm volatile("" ::"v"(sink));  // the touched words are used, so the loads stay
-      return;
-    }
-  }
 #pragma unroll
   for (int s0 = 0; s0 < NS - 1; ++s0) {
     if (s0 < nt) issue(s0, s0);
   }
+  // stage 0 has to be there before anything is read
+  if (nt > 1) {
+    wait_vmcnt<(NS - 2) * (PA + PB)>();  // with nt < NS - 1 fewer requests exist: the wait is merely stricter
+  } else {
+    wait_vmcnt<0>();
+  }
+  asm volatile("s_barrier" ::: "memory");
+  read_frags(0, 0, 0);
   int slot = 0, fill = NS - 1;  // ring slots of stage t and of stage t + NS - 1
+  auto next_of = [](int v) { return v + 1 == NS ? 0 : v + 1; };
   const int n_main = max(nt - (NS - 1), 0);
   for (int t = 0; t < n_main; ++t) {
-    // stages t+1 .. t+NS-2 may stay in flight; stage t must have landed
-    wait_vmcnt<(NS - 2) * (PA + PB)>();
-    // a bare barrier: __syncthreads() would first wait for every outstanding load, the requests
-    // for the stages ahead included.  No LDS store is pending here (the loop has none) and the
-    // LDS reads of the previous stage were consumed by its matrix instructions.
-    asm volatile("s_barrier" ::: "memory");
-    compute(slot, std::true_type{}, t + NS - 1, fill);
-    slot = slot + 1 == NS ? 0 : slot + 1;
-    fill = fill + 1 == NS ? 0 : fill + 1;
+    // after this stage's requests (stage t+NS-1), stages t+2 .. t+NS-1 may stay in flight when
+    // stage t+1 must have landed
+    stage(slot, std::true_type{}, t + NS - 1, fill, std::true_type{}, std::integral_constant<int, (NS - 2) * (PA + PB)>{},
+          next_of(slot));
+    slot = next_of(slot);
+    fill = next_of(fill);
   }
   // the last NS-1 stages: nothing left to request, so simply wait for everything
   for (int t = n_main; t < nt; ++t) {
-    wait_vmcnt<0>();
-    asm volatile("s_barrier" ::: "memory");
-    compute(slot, std::false_type{}, 0, 0);
-    slot = slot + 1 == NS ? 0 : slot + 1;
+    if (t + 1 < nt) {
+      stage(slot, std::false_type{}, 0, 0, std::true_type{}, std::integral_constant<int, 0>{}, next_of(slot));
+    } else {
+      stage(slot, std::false_type{}, 0, 0, std::false_type{}, std::integral_constant<int, 0>{}, 0);
+    }
+    slot = next_of(slot);
   }
   __syncthreads();  // the last stage has been read by everybody: LDS is free for the partial sums
 
@@ -566,13 +570,13 @@ __global__ __launch_bounds__(64 * (WM * WN * KS + (PF > 0 ? 1 : 0)), WM * WN * K
   }
 }
 
-template <int BM, int BN, int WM, int WN, int KS, int NS, int PF>
+template <int BM, int BN, int WM, int WN, int KS, int NS>
 int launch_dl(half_t* out, const half_t* A, const half_t* W, int M, int K, int N, float beta, hipStream_t st) {
   constexpr size_t lds = (size_t)NS * (BM + BN) * (BK * KS * 2);
   static_assert(lds <= 160 * 1024, "ring does not fit LDS");
   static_assert(KS == 1 || lds >= (size_t)BM * BN * 4 / 2, "LDS must hold one group's accumulators");
   const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
-  auto kernel = gemm_dl_kernel<BM, BN, WM, WN, KS, NS, PF>;
+  auto kernel = gemm_dl_kernel<BM, BN, WM, WN, KS, NS>;
   if constexpr (lds > 64 * 1024) {
     static bool raised[16] = {};  // per device, once
     int dev = 0;
@@ -582,7 +586,7 @@ int launch_dl(half_t* out, const half_t* A, const half_t* W, int M, int K, int N
       raised[dev & 15] = true;
     }
   }
-  kernel<<<tiles_m * tiles_n, 64 * (WM * WN * KS + (PF > 0 ? 1 : 0)), lds, st>>>(out, A, W, M, K, N, beta, tiles_m, tiles_n);
+  kernel<<<tiles_m * tiles_n, 64 * WM * WN * KS, lds, st>>>(out, A, W, M, K, N, beta, tiles_m, tiles_n);
   LCU_LAUNCH_CHECK();
   return LCU_OK;
 }
@@ -634,9 +638,9 @@ int dispatch_gemm(half_t* out, const half_t* A, const void* W, const half_t* S, 
   if constexpr (!U8) {
     if (K % 128 == 0) {  // fp16 weights, whole stages: the direct-to-LDS kernels
       const long tiles256 = (long)((M + 255) / 256) * ((N + 127) / 128);
-      if (tiles256 >= 160) return launch_dl<256, 128, 4, 2, 1, 3, 0>(out, A, (const half_t*)W, M, K, N, beta, st);
-      if (tiles128 >= 256) return launch_dl<128, 128, 2, 2, 1, 2, 0>(out, A, (const half_t*)W, M, K, N, beta, st);
-      return launch_dl<128, 64, 2, 2, 2, 3, 0>(out, A, (const half_t*)W, M, K, N, beta, st);
+      if (tiles256 >= 160) return launch_dl<256, 128, 4, 2, 1, 3>(out, A, (const half_t*)W, M, K, N, beta, st);
+      if (tiles128 >= 256) return launch_dl<128, 128, 2, 2, 1, 2>(out, A, (const half_t*)W, M, K, N, beta, st);
+      return launch_dl<128, 64, 2, 2, 2, 3>(out, A, (const half_t*)W, M, K, N, beta, st);
     }
   }
   if (tiles128 >= 256) return launch_gemm<128, 128, U8, 1>(out, A, W, S, M, K, N, block, beta, st);

@@ -30,7 +30,7 @@ HBM_PEAK_GBS = 8000.0      # MI355X HBM3E
 # HBM bytes per launch of the dominant kernel from rocprofv3 FETCH_SIZE / WRITE_SIZE, scaled by a
 # 256 MiB copy kernel read under the same counters (FETCH_SIZE reads half the bytes here): see
 # profiles/decode_ffn_up_kernel_llama7b_hbm_traffic.txt.  Counters are not read in this script.
-MEASURED_TRAFFIC = {"llama7b_fp16": 180643635}
+MEASURED_TRAFFIC = {"llama7b_fp16": 180639539}
 MFMA_F16_PEAK_TF = 2500.0  # dense fp16
 
 WORKLOADS = {

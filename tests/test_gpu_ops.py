@@ -304,6 +304,26 @@ def test_argmax_first_maximum(gpu):
     G.release()
 
 
+def test_error_stats(gpu):
+    G = gpu
+    for n in (1, 255, 4096, 1 << 20, (1 << 22) + 77):
+        a = normal((n,), 8, 1, 1.0)
+        b = normal((n,), 8, 2, 1.0)
+        out = G.empty((3,), np.float32)
+        da, db = G.dev_keep(a), G.dev_keep(b)
+        G.B.check(G.L().lcu_error_stats(out.ptr, da.ptr, db.ptr, n, None))
+        got = G.host(out, (3,), np.float32)
+        want = O.error_stats(a, b)
+        assert got[1] == want[1]                                  # the largest difference is exact
+        assert np.allclose(got[[0, 2]], want[[0, 2]], rtol=1e-5)  # fp32 partial sums against double
+        # run to run identical (the reference's atomics are not)
+        G.B.check(G.L().lcu_error_stats(out.ptr, da.ptr, db.ptr, n, None))
+        assert (G.host(out, (3,), np.float32) == got).all()
+        G.B.check(G.L().lcu_error_stats(out.ptr, da.ptr, da.ptr, n, None))
+        assert (G.host(out, (3,), np.float32) == 0).all()
+        G.release()
+
+
 def test_memset_and_copies(gpu):
     G = gpu
     for n in (1, 15, 16, 17, 4099, 1 << 20):

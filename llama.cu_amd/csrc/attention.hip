@@ -12,9 +12,10 @@
 // Decode (n_new == 1): one 1024-thread workgroup per head does scores, softmax and the weighted
 // sum in one launch; 16 lanes share one cached row (16 bytes each), 64 rows per pass, 16 passes of
 // loads in flight per thread.
-// Prefill (n_new > 1), matrix-core bound: one workgroup per (32 query rows, head); Q.K^T by
-// v_mfma_f32_16x16x32_f16 into an LDS score strip [32][T], softmax in LDS, P.V by MFMA with V
-// staged transposed in LDS.
+// Prefill (n_new > 1), matrix-core bound: one workgroup per (16 or 32 query rows, head); Q.K^T by
+// v_mfma_f32_16x16x32_f16 into an LDS score strip [rows][T], softmax in LDS, P.V by MFMA with V
+// staged row-major in LDS; the next 64-row chunk of K or V is in flight while the current one is
+// multiplied.
 #include "common.hpp"
 
 using namespace lcu;
@@ -148,19 +149,23 @@ __global__ __launch_bounds__(DEC_THREADS) void decode_attention_kernel(half_t* _
 // ---------------------------------------------------------------------------------------------
 // prefill
 // ---------------------------------------------------------------------------------------------
-constexpr int BR = 32;         // query rows per workgroup
 constexpr int CW = 64;         // cache rows per staged chunk
 constexpr int QLD = HD + 8;    // LDS row stride (halves) of the Q and K tiles
-constexpr int VLD = CW + 8;    // LDS row stride of the transposed V chunk
 constexpr int MAX_T_PREFILL = 2048;
 
+// BR: query rows per workgroup (16 or 32)
+template <int BR>
 __global__ __launch_bounds__(256) void prefill_attention_kernel(half_t* __restrict__ out, const half_t* __restrict__ q,
                                                                 const half_t* __restrict__ k, const half_t* __restrict__ v,
                                                                 int n_new, int T, int start_pos, int dim, int n_tiles) {
+  constexpr int RT = BR / 16;  // 16-row matrix-instruction tiles per workgroup
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-  // heavier (later) row tiles first: their causal span is longest
-  const int tile = n_tiles - 1 - blockIdx.x;
-  const int h = blockIdx.y;
+  // Heaviest work first over the whole grid (a later row tile has the longer causal span): the
+  // heads' last tiles, then their second-to-last ones, and so on, so that compute units pick up
+  // the short tiles as they run out of long ones instead of some holding only long ones.
+  const int n_heads = gridDim.x / n_tiles;
+  const int tile = n_tiles - 1 - blockIdx.x / n_heads;
+  const int h = blockIdx.x % n_heads;
   const int r0 = tile * BR;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   // columns this tile can see: c <= r + start_pos for its last real row
@@ -170,8 +175,8 @@ __global__ __launch_bounds__(256) void prefill_attention_kernel(half_t* __restri
   const int SLD = Tc + 8;
 
   half_t* Qs = reinterpret_cast<half_t*>(smem);             // [BR][QLD]
-  half_t* KVs = Qs + BR * QLD;                              // K chunk [CW][QLD] or V^T chunk [HD][VLD]
-  half_t* Ss = KVs + (CW * QLD > HD * VLD ? CW * QLD : HD * VLD);  // [BR][SLD]
+  half_t* KVs = Qs + BR * QLD;                              // K or V chunk [CW][QLD]
+  half_t* Ss = KVs + CW * QLD;                              // [BR][SLD]
 
   // Q tile
   for (int c = tid; c < BR * HD / 8; c += 256) {
@@ -184,23 +189,63 @@ __global__ __launch_bounds__(256) void prefill_attention_kernel(half_t* __restri
 
   const float denom = sqrtf((float)HD);
   const int frow = lane & 15, fk = (lane >> 4) * 8;
-  // ---- scores: S[BR][Tc] = Q . K^T, wave w owns the 16 columns w*16.. of every 64-column chunk
-  for (int c0 = 0; c0 < Tc; c0 += CW) {
-    __syncthreads();
-    for (int c = tid; c < CW * HD / 8; c += 256) {
-      const int row = c >> 4, col = (c & 15) * 8;
-      const int gp = c0 + row;
-      half8_t val = (half8_t)(0.0f);
-      if (gp < T) val = *reinterpret_cast<const half8_t*>(k + (size_t)gp * dim + h * HD + col);
-      *reinterpret_cast<half8_t*>(&KVs[row * QLD + col]) = val;
+  // A chunk of 64 cache rows is 64 x 128 halves = 4 x 16 bytes per thread.  The next chunk is
+  // requested into registers before the current one is multiplied, so its latency hides behind
+  // the matrix instructions instead of standing between two barriers.
+  constexpr int CH = CW * HD / 8 / 256;  // 16-byte pieces per thread and chunk
+  auto load_chunk = [&](half8_t (&reg)[CH], const half_t* __restrict__ src, int c0) {
+#pragma unroll
+    for (int i = 0; i < CH; ++i) {
+      const int c = tid + i * 256;
+      const int gp = min(c0 + (c >> 4), T - 1);  // rows past T are never used: their scores are masked, their P is 0
+      reg[i] = *reinterpret_cast<const half8_t*>(src + (size_t)gp * dim + h * HD + (c & 15) * 8);
     }
-    __syncthreads();
-    float4_t acc[2] = {(float4_t)(0.0f), (float4_t)(0.0f)};
+  };
+  auto store_chunk = [&](const half8_t (&reg)[CH]) {
+#pragma unroll
+    for (int i = 0; i < CH; ++i) {
+      const int c = tid + i * 256;
+      *reinterpret_cast<half8_t*>(&KVs[(c >> 4) * QLD + (c & 15) * 8]) = reg[i];
+    }
+  };
+
+  // Three chunks are in flight in registers: one chunk's matrix work is far shorter than a
+  // global load, so a single chunk of look-ahead leaves the load latency exposed.
+  constexpr int NPF = 3;
+  half8_t stage[NPF][CH];
+  auto for_chunks = [&](const half_t* __restrict__ src, auto&& body) {
+    for (int c0 = 0; c0 < Tc; c0 += NPF * CW) {
+#pragma unroll
+      for (int j = 0; j < NPF; ++j) {
+        const int cc = c0 + j * CW;
+        if (cc < Tc) {
+          __syncthreads();  // everybody is done with the previous chunk
+          store_chunk(stage[j]);
+          __syncthreads();
+          if (cc + NPF * CW < Tc) load_chunk(stage[j], src, cc + NPF * CW);
+          body(cc);
+        }
+      }
+    }
+  };
+  auto prefetch_first = [&](const half_t* __restrict__ src) {
+#pragma unroll
+    for (int j = 0; j < NPF; ++j) {
+      if (j * CW < Tc) load_chunk(stage[j], src, j * CW);
+    }
+  };
+
+  // ---- scores: S[BR][Tc] = Q . K^T, wave w owns the 16 columns w*16.. of every 64-column chunk
+  prefetch_first(k);
+  for_chunks(k, [&](int c0) {
+    float4_t acc[RT];
+#pragma unroll
+    for (int i = 0; i < RT; ++i) acc[i] = (float4_t)(0.0f);
 #pragma unroll
     for (int ks = 0; ks < HD; ks += 32) {
       const half8_t fb = *reinterpret_cast<const half8_t*>(&KVs[(wave * 16 + frow) * QLD + ks + fk]);
 #pragma unroll
-      for (int i = 0; i < 2; ++i) {
+      for (int i = 0; i < RT; ++i) {
         const half8_t fa = *reinterpret_cast<const half8_t*>(&Qs[(i * 16 + frow) * QLD + ks + fk]);
         acc[i] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fa, fb, acc[i], 0, 0, 0);
       }
@@ -208,64 +253,70 @@ __global__ __launch_bounds__(256) void prefill_attention_kernel(half_t* __restri
     // accumulator register e of lane l is (row 4*(l/16) + e, column l%16)
     const int col = c0 + wave * 16 + (lane & 15);
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
+    for (int i = 0; i < RT; ++i) {
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
         const int row = i * 16 + (lane >> 4) * 4 + e;
-        const bool masked = col > r0 + row + start_pos;  // llama_cu.cu:415
+        const bool masked = col > r0 + row + start_pos || col >= T;  // llama_cu.cu:415
         Ss[row * SLD + col] = masked ? (half_t)(-INFINITY) : round_f16(acc[i][e] / denom);
       }
     }
-  }
+  });
+  // the first V chunks travel while the softmax runs
+  prefetch_first(v);
   __syncthreads();
 
-  // ---- softmax over each row of the strip (llama_cu.cu:433-499): wave w owns rows w*8 .. w*8+7
+  // ---- softmax over each row of the strip (llama_cu.cu:433-499): wave w owns rows w*8 .. w*8+7.
+  // exp is v_exp_f32 on x * log2(e) and the division a reciprocal multiply (both within an fp32
+  // ulp or two of the library calls, far below the fp16 rounding of the result): with the library
+  // expf the softmax was the longest phase of the kernel.
+  constexpr float LOG2E = 1.4426950408889634f;
   for (int rr = 0; rr < BR / 4; ++rr) {
     half_t* srow = Ss + (wave * (BR / 4) + rr) * SLD;
     float m = -INFINITY;
     for (int i = lane; i < Tc; i += WAVE) m = fmaxf(m, (float)srow[i]);
     m = wave_max(m);
+    const float m2 = m * LOG2E;
     float s = 0.0f;
-    for (int i = lane; i < Tc; i += WAVE) s += expf((float)srow[i] - m);
+    for (int i = lane; i < Tc; i += WAVE) s += __builtin_amdgcn_exp2f(fmaf((float)srow[i], LOG2E, -m2));
     s = wave_sum(s);
-    for (int i = lane; i < Tc; i += WAVE) srow[i] = round_f16(expf((float)srow[i] - m) / s);
+    const float inv = __builtin_amdgcn_rcpf(s);
+    for (int i = lane; i < Tc; i += WAVE) {
+      srow[i] = round_f16(__builtin_amdgcn_exp2f(fmaf((float)srow[i], LOG2E, -m2)) * inv);
+    }
   }
 
   // ---- out[BR][HD] = P . V: wave w owns output columns w*32 .. w*32+31 (two 16-wide tiles)
-  float4_t o[2][2];
+  float4_t o[RT][2];
 #pragma unroll
-  for (int i = 0; i < 2; ++i) {
+  for (int i = 0; i < RT; ++i) {
 #pragma unroll
     for (int j = 0; j < 2; ++j) o[i][j] = (float4_t)(0.0f);
   }
-  for (int c0 = 0; c0 < Tc; c0 += CW) {
-    __syncthreads();
-    // V chunk, transposed on the way into LDS: KVs[d][pos]
-    for (int c = tid; c < CW * HD / 8; c += 256) {
-      const int row = c >> 4, col = (c & 15) * 8;
-      const int gp = c0 + row;
-      half8_t val = (half8_t)(0.0f);
-      if (gp < T) val = *reinterpret_cast<const half8_t*>(v + (size_t)gp * dim + h * HD + col);
-#pragma unroll
-      for (int e = 0; e < 8; ++e) KVs[(col + e) * VLD + row] = val[e];
-    }
-    __syncthreads();
+  // V chunks stay row-major in LDS, KVs[pos][d] (16-byte stores without bank conflicts); the
+  // matrix instruction wants 8 consecutive positions of one output column per lane, which are
+  // gathered with 2-byte reads: the 16 lanes of a fragment row group read 16 neighbouring columns.
+  for_chunks(v, [&](int c0) {
 #pragma unroll
     for (int ks = 0; ks < CW; ks += 32) {
-      half8_t fa[2], fb[2];
+      half8_t fa[RT], fb[2];
 #pragma unroll
-      for (int i = 0; i < 2; ++i) fa[i] = *reinterpret_cast<const half8_t*>(&Ss[(i * 16 + frow) * SLD + c0 + ks + fk]);
+      for (int i = 0; i < RT; ++i) fa[i] = *reinterpret_cast<const half8_t*>(&Ss[(i * 16 + frow) * SLD + c0 + ks + fk]);
 #pragma unroll
-      for (int j = 0; j < 2; ++j) fb[j] = *reinterpret_cast<const half8_t*>(&KVs[(wave * 32 + j * 16 + frow) * VLD + ks + fk]);
+      for (int j = 0; j < 2; ++j) {
+        const half_t* vcol = &KVs[(ks + fk) * QLD + wave * 32 + j * 16 + frow];
 #pragma unroll
-      for (int i = 0; i < 2; ++i) {
+        for (int e = 0; e < 8; ++e) fb[j][e] = vcol[e * QLD];
+      }
+#pragma unroll
+      for (int i = 0; i < RT; ++i) {
 #pragma unroll
         for (int j = 0; j < 2; ++j) o[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fa[i], fb[j], o[i][j], 0, 0, 0);
       }
     }
-  }
+  });
 #pragma unroll
-  for (int i = 0; i < 2; ++i) {
+  for (int i = 0; i < RT; ++i) {
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
       const int col = h * HD + wave * 32 + j * 16 + (lane & 15);
@@ -278,8 +329,8 @@ __global__ __launch_bounds__(256) void prefill_attention_kernel(half_t* __restri
   }
 }
 
-size_t prefill_lds_bytes(int Tc) {
-  const size_t kv = (size_t)(CW * QLD > HD * VLD ? CW * QLD : HD * VLD);
+size_t prefill_lds_bytes(int BR, int Tc) {
+  const size_t kv = (size_t)CW * QLD;
   return ((size_t)BR * QLD + kv + (size_t)BR * (Tc + 8)) * sizeof(half_t);
 }
 
@@ -307,20 +358,33 @@ int lcu_attention(void* out_dev, const void* q_dev, const void* k_dev, const voi
     return LCU_OK;
   }
   LCU_REQUIRE(T <= MAX_T_PREFILL, "lcu_attention: T %d exceeds %d for n_new > 1", T, MAX_T_PREFILL);
+  // 16-row tiles when 32-row tiles would leave the grid under four workgroups per compute unit
+  // and the rows are short (T <= 1024: 22 us against 29 us at n = T = 512, dim 4096); with long
+  // rows the per-chunk overhead of the extra workgroups costs more than the balance gains.
+  const long wgs32 = (long)((n_new + 31) / 32) * n_heads;
+  const int BR = (wgs32 < 1024 && T <= 1024) ? 16 : 32;
   const int n_tiles = (n_new + BR - 1) / BR;
   const int Tc_max = (T + CW - 1) / CW * CW;
-  const size_t lds = prefill_lds_bytes(Tc_max);
+  const size_t lds = prefill_lds_bytes(BR, Tc_max);
   static bool attr_set[16] = {};
   int dev = 0;
   LCU_HIP(hipGetDevice(&dev));
   if (!attr_set[dev & 15]) {
-    LCU_HIP(hipFuncSetAttribute((const void*)prefill_attention_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                (int)prefill_lds_bytes(MAX_T_PREFILL)));
+    LCU_HIP(hipFuncSetAttribute((const void*)prefill_attention_kernel<16>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                (int)prefill_lds_bytes(16, MAX_T_PREFILL)));
+    LCU_HIP(hipFuncSetAttribute((const void*)prefill_attention_kernel<32>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                (int)prefill_lds_bytes(32, MAX_T_PREFILL)));
     attr_set[dev & 15] = true;
   }
-  dim3 grid(n_tiles, n_heads);
-  prefill_attention_kernel<<<grid, 256, lds, s>>>((half_t*)out_dev, (const half_t*)q_dev, (const half_t*)k_dev,
-                                                  (const half_t*)v_dev, n_new, T, start_pos, dim, n_tiles);
+  if (BR == 16) {
+    prefill_attention_kernel<16><<<n_tiles * n_heads, 256, lds, s>>>(
+        (half_t*)out_dev, (const half_t*)q_dev, (const half_t*)k_dev, (const half_t*)v_dev, n_new, T, start_pos, dim,
+        n_tiles);
+  } else {
+    prefill_attention_kernel<32><<<n_tiles * n_heads, 256, lds, s>>>(
+        (half_t*)out_dev, (const half_t*)q_dev, (const half_t*)k_dev, (const half_t*)v_dev, n_new, T, start_pos, dim,
+        n_tiles);
+  }
   LCU_LAUNCH_CHECK();
   return LCU_OK;
 }

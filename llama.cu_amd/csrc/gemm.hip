@@ -327,23 +327,39 @@ __device__ __forceinline__ void wait_vmcnt() {
 // Tried and dropped: an extra wavefront that touches the lines of a stage several stages ahead so
 // that the loaders hit L2.  About a sixth of the requests come from HBM, but the touches (64
 // separate lines per instruction) cost the texture addresser more than the misses cost the ring.
-template <int BM, int BN, int WM, int WN, int KS, int NS>
+//
+// uint8 weights (U8): the codes travel the same way, into a ring of their own, one stage further
+// ahead than the lhs tile ("batch" b of requests = lhs of stage b + codes of stage b+1).  During
+// stage t the workgroup turns the codes of stage t+1 into the fp16 tile the matrix instructions
+// read -- every thread one 16-code chunk, each weight exactly fp16((q - 127.5) * scale), written
+// at the same permuted chunk positions a direct fp16 load would have filled -- so a weight is
+// dequantised once per block tile and the fragment path is the fp16 one.  The chunk's scale comes
+// by an ordinary 2-byte load one stage earlier.
+template <int BM, int BN, int WM, int WN, int KS, int NS, bool U8>
 __global__ __launch_bounds__(64 * WM * WN * KS, WM * WN * KS <= 4 ? 2 : 1) void gemm_dl_kernel(
-    half_t* __restrict__ out, const half_t* __restrict__ A, const half_t* __restrict__ W, int M, int K, int N,
-    float beta, int tiles_m, int tiles_n) {
+    half_t* __restrict__ out, const half_t* __restrict__ A, const void* __restrict__ W, const half_t* __restrict__ S,
+    int M, int K, int N, int block, float beta, int tiles_m, int tiles_n) {
   constexpr int NG = WM * WN;                // wavefronts of one group
   constexpr int NW = NG * KS;                // wavefronts
   constexpr int BKS = BK * KS;               // K extent of a stage
   constexpr int ROWB = BKS * 2;              // bytes of a tile row in LDS
   constexpr int CR = ROWB / 16;              // 16-byte chunks per row: 8 or 16
   constexpr int RPB = 16 / CR;               // tile rows per 256 bytes (one pass over the banks)
+  constexpr int THREADS = 64 * NW;
+  constexpr int CPR = BKS / 16;              // 16-code chunks per row of the code tile
   constexpr int PA = BM * CR / 64 / NW;      // load instructions per wavefront per stage, lhs
-  constexpr int PB = BN * CR / 64 / NW;      // and W
-  constexpr int A_BYTES = BM * ROWB;
-  constexpr int STAGE = (BM + BN) * ROWB;
+  constexpr int PB = U8 ? BN * CPR / 64 / NW : BN * CR / 64 / NW;  // and W (fp16 values or codes)
+  constexpr int DC = U8 ? BN * CPR / THREADS : 1;                  // code chunks a thread dequantises per stage
+  constexpr int A_BYTES = BM * ROWB, B_BYTES = BN * ROWB, C_BYTES = BN * BKS;
+  constexpr int NB = U8 ? 2 : NS;            // fp16 W tiles held: written one stage ahead, or the ring itself
+  // fp16: slot s of the ring holds lhs and W tile of a stage side by side; uint8: lhs ring, then the
+  // two fp16 W tiles, then the code ring
+  constexpr int A_STRIDE = U8 ? A_BYTES : A_BYTES + B_BYTES, B_STRIDE = U8 ? B_BYTES : A_BYTES + B_BYTES;
+  constexpr int B_BASE = U8 ? NS * A_BYTES : A_BYTES, C_BASE = NS * A_BYTES + NB * B_BYTES;
   constexpr int TM = BM / (32 * WM), TN = BN / (32 * WN);
-  static_assert(PA >= 1 && PB >= 1 && NS >= 2 && NS <= 4, "unsupported configuration");
-  static_assert((PA + PB) * (NS - 1) < 64, "vmcnt has 6 bits");
+  static_assert(PA >= 1 && PB >= 1 && DC >= 1 && NS >= 2 && NS <= 4, "unsupported configuration");
+  static_assert(!U8 || NS == 3, "the uint8 schedule is written for a ring of three");
+  static_assert((PA + PB + DC) * (NS - 1) < 64, "vmcnt has 6 bits");
 
   extern __shared__ __attribute__((aligned(16))) unsigned char gemm_lds[];
 
@@ -372,22 +388,33 @@ __global__ __launch_bounds__(64 * WM * WN * KS, WM * WN * KS <= 4 ? 2 : 1) void 
 #pragma unroll
   for (int j = 0; j < PB; ++j) {
     const int c = (wave + j * NW) * 64 + lane;
-    const int row = c / CR, g = (c % CR) ^ ((row / RPB) % CR);
-    b_off[j] = ((uint32_t)min(n0 + row, N - 1) * (uint32_t)K + g * 8) * 2u;
+    if constexpr (U8) {  // codes lie densely and unpermuted: chunk c of the tile at byte 16 c
+      b_off[j] = (uint32_t)min(n0 + c / CPR, N - 1) * (uint32_t)K + (c % CPR) * 16;
+    } else {
+      const int row = c / CR, g = (c % CR) ^ ((row / RPB) % CR);
+      b_off[j] = ((uint32_t)min(n0 + row, N - 1) * (uint32_t)K + g * 8) * 2u;
+    }
   }
   const char* Ab = (const char*)A;
   const char* Wb = (const char*)W;
   using gptr = const __attribute__((address_space(1))) void*;
   using lptr = __attribute__((address_space(3))) void*;
-  // load instruction `idx` (0 .. PA+PB-1) of this wavefront for K stage `stage` into ring slot `slot`
+  const int nt = K / BKS;
+  // load instruction `idx` (0 .. PA+PB-1) of this wavefront for batch `stage` into ring slot `slot`:
+  // the lhs tile of that stage, and the W tile of that stage (fp16) or the codes of the stage after
+  // it (uint8; past the end the last stage is fetched again and never used)
   auto issue_one = [&](int stage, int slot, int idx) {
-    const size_t kb = (size_t)stage * (BKS * 2);
-    unsigned char* base = gemm_lds + slot * STAGE + wave * 1024;
     if (idx < PA) {
-      __builtin_amdgcn_global_load_lds((gptr)(Ab + kb + a_off[idx]), (lptr)(base + idx * NW * 1024), 16, 0, 0);
+      unsigned char* dst = gemm_lds + slot * A_STRIDE + (wave + idx * NW) * 1024;
+      __builtin_amdgcn_global_load_lds((gptr)(Ab + (size_t)stage * (BKS * 2) + a_off[idx]), (lptr)dst, 16, 0, 0);
+    } else if constexpr (U8) {
+      const int cslot = slot + 1 == NS ? 0 : slot + 1;
+      unsigned char* dst = gemm_lds + C_BASE + cslot * C_BYTES + (wave + (idx - PA) * NW) * 1024;
+      __builtin_amdgcn_global_load_lds((gptr)(Wb + (size_t)min(stage + 1, nt - 1) * BKS + b_off[idx - PA]), (lptr)dst, 16,
+                                       0, 0);
     } else {
-      __builtin_amdgcn_global_load_lds((gptr)(Wb + kb + b_off[idx - PA]), (lptr)(base + A_BYTES + (idx - PA) * NW * 1024),
-                                       16, 0, 0);
+      unsigned char* dst = gemm_lds + B_BASE + slot * B_STRIDE + (wave + (idx - PA) * NW) * 1024;
+      __builtin_amdgcn_global_load_lds((gptr)(Wb + (size_t)stage * (BKS * 2) + b_off[idx - PA]), (lptr)dst, 16, 0, 0);
     }
   };
   auto issue = [&](int stage, int slot) {
@@ -412,7 +439,53 @@ __global__ __launch_bounds__(64 * WM * WN * KS, WM * WN * KS <= 4 ? 2 : 1) void 
   uint32_t pos[BK / 16];
 #pragma unroll
   for (int s4 = 0; s4 < BK / 16; ++s4) pos[s4] = (uint32_t)(((gbase + 2 * s4) ^ fr) * 16);
-  const uint32_t a_row = (uint32_t)(wm + frag_row) * ROWB, b_row = (uint32_t)A_BYTES + (uint32_t)(wn + frag_row) * ROWB;
+  const uint32_t a_row = (uint32_t)(wm + frag_row) * ROWB, b_row = (uint32_t)B_BASE + (uint32_t)(wn + frag_row) * ROWB;
+
+  // uint8: the chunks this thread dequantises (tile row, chunk in the row), their scale index at
+  // stage 0, and where the two fp16 chunks of a dequantised chunk go in the W tile
+  int d_scale[DC];
+  uint32_t d_src[DC], d_dst0[DC], d_dst1[DC];
+  half_t sc_cur[DC], sc_nxt[DC];
+  const int nblk = U8 ? K / block : 0;
+  if constexpr (U8) {
+#pragma unroll
+    for (int i = 0; i < DC; ++i) {
+      const int c = tid + i * THREADS;
+      const int row = c / CPR, kc = c % CPR, f = (row / RPB) % CR;
+      d_scale[i] = min(n0 + row, N - 1) * nblk;
+      d_src[i] = (uint32_t)c * 16;
+      d_dst0[i] = (uint32_t)row * ROWB + (uint32_t)(((2 * kc) ^ f) * 16);
+      d_dst1[i] = (uint32_t)row * ROWB + (uint32_t)(((2 * kc + 1) ^ f) * 16);
+    }
+  }
+  auto load_scales = [&](half_t (&sc)[DC], int stage) {
+    const int st = min(stage, nt - 1);
+#pragma unroll
+    for (int i = 0; i < DC; ++i) {
+      const int kc = (tid + i * THREADS) % CPR;
+      sc[i] = S[d_scale[i] + (st * BKS + kc * 16) / block];
+    }
+  };
+  // codes in ring slot `cslot` -> fp16 W tile `bslot`
+  auto dequantise = [&](int cslot, int bslot, const half_t (&sc)[DC]) {
+#pragma unroll
+    for (int i = 0; i < DC; ++i) {
+      const uint4_t q = *reinterpret_cast<const uint4_t*>(gemm_lds + C_BASE + cslot * C_BYTES + d_src[i]);
+      const half_t s2 = sc[i] * (half_t)2.0f;
+      const half2_t s2v = {s2, s2};
+      half2_t d[8];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        d[2 * j] = dequant2(__builtin_amdgcn_perm(0u, q[j], 0x0c010c00u), s2v);
+        d[2 * j + 1] = dequant2(__builtin_amdgcn_perm(0u, q[j], 0x0c030c02u), s2v);
+      }
+      const half8_t lo = {d[0].x, d[0].y, d[1].x, d[1].y, d[2].x, d[2].y, d[3].x, d[3].y};
+      const half8_t hi = {d[4].x, d[4].y, d[5].x, d[5].y, d[6].x, d[6].y, d[7].x, d[7].y};
+      unsigned char* tile = gemm_lds + B_BASE + bslot * B_STRIDE;
+      *reinterpret_cast<half8_t*>(tile + d_dst0[i]) = lo;
+      *reinterpret_cast<half8_t*>(tile + d_dst1[i]) = hi;
+    }
+  };
 
   // ---- the stage loop, scheduled by hand ------------------------------------------------------
   // The LDS reads and their waits are written as inline assembly: with global_load_lds requests
@@ -432,8 +505,8 @@ __global__ __launch_bounds__(64 * WM * WN * KS, WM * WN * KS <= 4 ? 2 : 1) void 
   static_assert(S4 == 4, "the schedule below is written for four K slices per stage");
   const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char*)gemm_lds;
   half8_t fa[2][TM], fb[2][TN];
-  auto read_frags = [&](int buf, int slot, int s4) {
-    const uint32_t pa = lds0 + slot * STAGE + a_row + pos[s4], pb = lds0 + slot * STAGE + b_row + pos[s4];
+  auto read_frags = [&](int buf, int slot, int bslot, int s4) {
+    const uint32_t pa = lds0 + slot * A_STRIDE + a_row + pos[s4], pb = lds0 + bslot * B_STRIDE + b_row + pos[s4];
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
       asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(fa[buf][i]) : "v"(pa), "n"(i * 32 * ROWB));
@@ -459,14 +532,20 @@ __global__ __launch_bounds__(64 * WM * WN * KS, WM * WN * KS <= 4 ? 2 : 1) void 
       }
     }
   };
-  // one stage; FETCH: request stage `next` into slot `fill`; MORE: another stage follows (in
-  // `nslot`), whose own requests are complete once at most PEND requests are outstanding
-  auto stage = [&](int slot, auto fetch, int next, int fill, auto more, auto pend, int nslot) {
+  // one stage (lhs in ring slot `slot`, W tile `bslot`); FETCH: request batch `next` into slot
+  // `fill`; MORE: another stage follows (slots `nslot`, `nbslot`), whose own requests are complete
+  // once at most PEND younger ones are outstanding.  uint8 with MORE: the scales of the stage after
+  // the next are requested first, and between the first two slices the codes of the next stage
+  // (ring slot nslot) become its fp16 tile nbslot.  Those LDS accesses are the compiler's; being
+  // younger than the fragments a slice waits for, they can only make the hand-counted waits stricter.
+  auto stage = [&](int slot, int bslot, auto fetch, int next, int fill, auto more, auto pend, int nslot, int nbslot,
+                   int t) {
     constexpr bool FETCH = decltype(fetch)::value, MORE = decltype(more)::value;
     constexpr int PEND = decltype(pend)::value;
+    if constexpr (U8 && MORE) load_scales(sc_nxt, t + 2);
 #pragma unroll
     for (int s4 = 0; s4 < 3; ++s4) {
-      read_frags((s4 + 1) & 1, slot, s4 + 1);
+      read_frags((s4 + 1) & 1, slot, bslot, s4 + 1);
       asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(TM + TN) : "memory");
       frags_ready(s4 & 1);
       if constexpr (FETCH) {
@@ -474,47 +553,76 @@ __global__ __launch_bounds__(64 * WM * WN * KS, WM * WN * KS <= 4 ? 2 : 1) void 
         for (int idx = s4 * P / 3; idx < (s4 + 1) * P / 3; ++idx) issue_one(next, fill, idx);
       }
       multiply(s4 & 1);
+      if constexpr (U8 && MORE) {
+        if (s4 == 0) dequantise(nslot, nbslot, sc_cur);
+      }
     }
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     frags_ready(1);
     if constexpr (MORE) {
       wait_vmcnt<PEND>();
       asm volatile("s_barrier" ::: "memory");
-      read_frags(0, nslot, 0);
+      read_frags(0, nslot, nbslot, 0);
     }
     multiply(1);
+    if constexpr (U8 && MORE) {
+#pragma unroll
+      for (int i = 0; i < DC; ++i) sc_cur[i] = sc_nxt[i];
+    }
   };
 
-  const int nt = K / BKS;
+  constexpr int PS = U8 ? P + DC : P;  // vector-memory requests per stage: the batch, and the scale loads
+  if constexpr (U8) {
+    // scales of stages 0 and 1, codes of stage 0 (into code slot 0), then the first batches
+    half_t sc0[DC];
+    load_scales(sc0, 0);
+    load_scales(sc_cur, 1);
 #pragma unroll
-  for (int s0 = 0; s0 < NS - 1; ++s0) {
-    if (s0 < nt) issue(s0, s0);
+    for (int idx = PA; idx < P; ++idx) issue_one(-1, NS - 1, idx);
+#pragma unroll
+    for (int s0 = 0; s0 < NS - 1; ++s0) {
+      if (s0 < nt) issue(s0, s0);
+    }
+    if (nt > 1) {
+      wait_vmcnt<(NS - 1) * P>();  // everything older than the batches: the codes of stage 0
+    } else {
+      wait_vmcnt<0>();
+    }
+    asm volatile("s_barrier" ::: "memory");
+    dequantise(0, 0, sc0);
+  } else {
+#pragma unroll
+    for (int s0 = 0; s0 < NS - 1; ++s0) {
+      if (s0 < nt) issue(s0, s0);
+    }
   }
   // stage 0 has to be there before anything is read
   if (nt > 1) {
-    wait_vmcnt<(NS - 2) * (PA + PB)>();  // with nt < NS - 1 fewer requests exist: the wait is merely stricter
+    wait_vmcnt<(NS - 2) * P>();  // with nt < NS - 1 fewer requests exist: the wait is merely stricter
   } else {
     wait_vmcnt<0>();
   }
-  asm volatile("s_barrier" ::: "memory");
-  read_frags(0, 0, 0);
-  int slot = 0, fill = NS - 1;  // ring slots of stage t and of stage t + NS - 1
+  __syncthreads();  // also orders the fp16 tile written just above (uint8) before its first reads
+  read_frags(0, 0, 0, 0);
+  int slot = 0, fill = NS - 1;  // ring slots of stage t and of batch t + NS - 1
   auto next_of = [](int v) { return v + 1 == NS ? 0 : v + 1; };
   const int n_main = max(nt - (NS - 1), 0);
   for (int t = 0; t < n_main; ++t) {
-    // after this stage's requests (stage t+NS-1), stages t+2 .. t+NS-1 may stay in flight when
-    // stage t+1 must have landed
-    stage(slot, std::true_type{}, t + NS - 1, fill, std::true_type{}, std::integral_constant<int, (NS - 2) * (PA + PB)>{},
-          next_of(slot));
+    // after this stage's requests (batch t+NS-1 and, uint8, scale loads), stages t+2 .. t+NS-1 may
+    // stay in flight when stage t+1 must have landed
+    stage(slot, U8 ? (t & 1) : slot, std::true_type{}, t + NS - 1, fill, std::true_type{},
+          std::integral_constant<int, (NS - 2) * PS>{}, next_of(slot), U8 ? ((t + 1) & 1) : next_of(slot), t);
     slot = next_of(slot);
     fill = next_of(fill);
   }
   // the last NS-1 stages: nothing left to request, so simply wait for everything
   for (int t = n_main; t < nt; ++t) {
     if (t + 1 < nt) {
-      stage(slot, std::false_type{}, 0, 0, std::true_type{}, std::integral_constant<int, 0>{}, next_of(slot));
+      stage(slot, U8 ? (t & 1) : slot, std::false_type{}, 0, 0, std::true_type{}, std::integral_constant<int, 0>{},
+            next_of(slot), U8 ? ((t + 1) & 1) : next_of(slot), t);
     } else {
-      stage(slot, std::false_type{}, 0, 0, std::false_type{}, std::integral_constant<int, 0>{}, 0);
+      stage(slot, U8 ? (t & 1) : slot, std::false_type{}, 0, 0, std::false_type{}, std::integral_constant<int, 0>{}, 0, 0,
+            t);
     }
     slot = next_of(slot);
   }
@@ -570,13 +678,15 @@ __global__ __launch_bounds__(64 * WM * WN * KS, WM * WN * KS <= 4 ? 2 : 1) void 
   }
 }
 
-template <int BM, int BN, int WM, int WN, int KS, int NS>
-int launch_dl(half_t* out, const half_t* A, const half_t* W, int M, int K, int N, float beta, hipStream_t st) {
-  constexpr size_t lds = (size_t)NS * (BM + BN) * (BK * KS * 2);
-  static_assert(lds <= 160 * 1024, "ring does not fit LDS");
+template <int BM, int BN, int WM, int WN, int KS, int NS, bool U8>
+int launch_dl(half_t* out, const half_t* A, const void* W, const half_t* S, int M, int K, int N, int block,
+              float beta, hipStream_t st) {
+  constexpr int ROWB = BK * KS * 2;
+  constexpr size_t lds = (size_t)NS * BM * ROWB + (size_t)(U8 ? 2 : NS) * BN * ROWB + (U8 ? (size_t)NS * BN * BK * KS : 0);
+  static_assert(lds <= 160 * 1024, "rings do not fit LDS");
   static_assert(KS == 1 || lds >= (size_t)BM * BN * 4 / 2, "LDS must hold one group's accumulators");
   const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
-  auto kernel = gemm_dl_kernel<BM, BN, WM, WN, KS, NS>;
+  auto kernel = gemm_dl_kernel<BM, BN, WM, WN, KS, NS, U8>;
   if constexpr (lds > 64 * 1024) {
     static bool raised[16] = {};  // per device, once
     int dev = 0;
@@ -586,7 +696,7 @@ int launch_dl(half_t* out, const half_t* A, const half_t* W, int M, int K, int N
       raised[dev & 15] = true;
     }
   }
-  kernel<<<tiles_m * tiles_n, 64 * WM * WN * KS, lds, st>>>(out, A, W, M, K, N, beta, tiles_m, tiles_n);
+  kernel<<<tiles_m * tiles_n, 64 * WM * WN * KS, lds, st>>>(out, A, W, S, M, K, N, block, beta, tiles_m, tiles_n);
   LCU_LAUNCH_CHECK();
   return LCU_OK;
 }
@@ -629,21 +739,30 @@ int launch_gemm(half_t* out, const half_t* A, const void* W, const half_t* S, in
 template <bool U8>
 int dispatch_gemm(half_t* out, const half_t* A, const void* W, const half_t* S, int M, int K, int N, int block,
                   float beta, hipStream_t st) {
-  // 128x128 tiles when there are enough of them to give every compute unit one (two fit a compute
-  // unit and desynchronise, which hides LDS latency better than the paired groups of KS = 2 do:
-  // 344 such tiles at N = 11008 beat 344 workgroups of eight wavefronts); else 128x64 tiles, of which there
-  // are then fewer than two per compute unit, so the workgroup brings the second group of
-  // wavefronts itself (M = 512, N = 4096: 35 us against 41 us, K = 11008: 100 us against 135 us).
+  // Tile choice.  Large tiles read fewer operand bytes per multiply-add, and the per-CU load path
+  // is what these kernels run against; but a compute unit needs two wavefronts per SIMD to overlap
+  // LDS waits with matrix work.  So: 256x128 tiles with eight wavefronts when that still gives 160
+  // workgroups (fp16 path); 128x128 with four when every compute unit gets one (two fit and
+  // desynchronise: 344 such tiles at N = 11008 beat 344 workgroups of eight wavefronts); 128x64
+  // with four wavefronts when there are more of them than compute units (two fit); else 128x64
+  // with two groups of four wavefronts splitting the K stage, because then the grid cannot give a
+  // compute unit a second workgroup (M = 512, N = 4096: 35 us against 41 us, K = 11008: 100 us
+  // against 135 us with the register-staged kernel).
   const long tiles128 = (long)((M + 127) / 128) * ((N + 127) / 128);
-  if constexpr (!U8) {
-    if (K % 128 == 0) {  // fp16 weights, whole stages: the direct-to-LDS kernels
-      const long tiles256 = (long)((M + 255) / 256) * ((N + 127) / 128);
-      if (tiles256 >= 160) return launch_dl<256, 128, 4, 2, 1, 3>(out, A, (const half_t*)W, M, K, N, beta, st);
-      if (tiles128 >= 256) return launch_dl<128, 128, 2, 2, 1, 2>(out, A, (const half_t*)W, M, K, N, beta, st);
-      return launch_dl<128, 64, 2, 2, 2, 3>(out, A, (const half_t*)W, M, K, N, beta, st);
+  const long tiles64 = (long)((M + 127) / 128) * ((N + 63) / 64);
+  if (K % 128 == 0) {  // whole stages: the direct-to-LDS kernels
+    const long tiles256 = (long)((M + 255) / 256) * ((N + 127) / 128);
+    if (tiles256 >= 160) return launch_dl<256, 128, 4, 2, 1, 3, U8>(out, A, W, S, M, K, N, block, beta, st);
+    if constexpr (!U8) {  // uint8 needs a code ring and two W tiles besides: too much LDS for two workgroups
+      if (tiles128 >= 256) return launch_dl<128, 128, 2, 2, 1, 2, false>(out, A, W, S, M, K, N, block, beta, st);
+    }
+    if (tiles128 < 256) {
+      if (tiles64 > 256) return launch_dl<128, 64, 2, 2, 1, 3, U8>(out, A, W, S, M, K, N, block, beta, st);
+      return launch_dl<128, 64, 2, 2, 2, 3, U8>(out, A, W, S, M, K, N, block, beta, st);
     }
   }
   if (tiles128 >= 256) return launch_gemm<128, 128, U8, 1>(out, A, W, S, M, K, N, block, beta, st);
+  if (tiles64 > 256) return launch_gemm<128, 64, U8, 1>(out, A, W, S, M, K, N, block, beta, st);
   return launch_gemm<128, 64, U8, 2>(out, A, W, S, M, K, N, block, beta, st);
 }
 

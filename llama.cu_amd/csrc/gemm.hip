@@ -757,6 +757,7 @@ int dispatch_gemm(half_t* out, const half_t* A, const void* W, const half_t* S, 
       if (tiles128 >= 256) return launch_dl<128, 128, 2, 2, 1, 2, false>(out, A, W, S, M, K, N, block, beta, st);
     }
     if (tiles128 < 256) {
+      if (tiles128 >= 160) return launch_dl<128, 128, 4, 2, 1, 3, U8>(out, A, W, S, M, K, N, block, beta, st);
       if (tiles64 > 256) return launch_dl<128, 64, 2, 2, 1, 3, U8>(out, A, W, S, M, K, N, block, beta, st);
       return launch_dl<128, 64, 2, 2, 2, 3, U8>(out, A, W, S, M, K, N, block, beta, st);
     }

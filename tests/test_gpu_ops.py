@@ -147,8 +147,12 @@ def test_gemv_u8_dequant_is_exact(gpu):
     G.release()
 
 
+# the shapes cover every tile configuration of the dispatcher: 128x64 with two wavefront groups,
+# 256x128, 128x128 with eight wavefronts (160..255 tiles: N = 5120), 128x64 with two workgroups per
+# compute unit (N = 4160), 128x128 with four wavefronts (M = 1024, N = 4096), and ragged K / M / N
 @pytest.mark.parametrize("M,K,N", [(512, 4096, 4096), (512, 4096, 11008), (512, 11008, 4096), (128, 256, 128),
-                                   (7, 64, 24), (130, 200, 70), (33, 1024, 257)])
+                                   (7, 64, 24), (130, 200, 70), (33, 1024, 257), (512, 256, 5120), (512, 384, 4160),
+                                   (1024, 256, 4096), (500, 128, 5100)])
 def test_gemm_f16(gpu, M, K, N):
     G = gpu
     x = normal((M, K), 0, 300, 1.0)
@@ -179,7 +183,8 @@ def test_gemm_exact_cases(gpu):
 
 
 @pytest.mark.parametrize("M,K,N", [(512, 4096, 4096), (512, 4096, 11008), (512, 11008, 4096), (16, 256, 128),
-                                   (130, 384, 70)])
+                                   (130, 384, 70), (512, 256, 5120), (512, 384, 4160), (1024, 256, 4096),
+                                   (500, 128, 5100), (40, 384, 300)])
 def test_gemm_u8(gpu, M, K, N):
     G = gpu
     x = normal((M, K), 0, 400, 1.0)

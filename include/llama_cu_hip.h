@@ -127,7 +127,10 @@ int lcu_attention(void* out_dev, const void* q_dev, const void* k_dev, const voi
                   int n_new, int T, int start_pos, int dim, int n_heads, void* stream);
 
 /* lcu_attention for one new token whose position (= T - 1) is read from the device int32 pos_dev
- * when the kernel runs; max_T bounds it (the cache length). */
+ * when the kernel runs; max_T bounds it (at most the cache length; the position is clamped to it).
+ * A bound of 1024 or less selects the single-launch kernel, a larger one the two-launch form that
+ * spreads long rows over the chip, so a caller that replays a captured graph keeps the bound at
+ * 1024 while the position allows it.  Uses the per-device workspace when max_T > 1024. */
 int lcu_attention_decode(void* out_dev, const void* q_dev, const void* k_dev, const void* v_dev,
                          const void* pos_dev, int max_T, int dim, int n_heads, void* stream);
 

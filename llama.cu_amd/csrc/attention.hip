@@ -9,8 +9,8 @@
 // Layouts: q [n_new, dim]; k, v = first T rows of a [*, dim] cache (K already rotated); head h is
 // columns h*128 .. h*128+127.
 //
-// Decode (n_new == 1): one 1024-thread workgroup per head does scores, softmax and the weighted
-// sum in one launch; 16 lanes share one cached row (16 bytes each), 64 rows per pass, 16 passes of
+// Decode (n_new == 1), up to 1024 cached rows: one 1024-thread workgroup per head does scores,
+// softmax and the weighted sum in one launch; beyond, two launches (see dec_scores_kernel); 16 lanes share one cached row (16 bytes each), 64 rows per pass, 16 passes of
 // loads in flight per thread.
 // Prefill (n_new > 1), matrix-core bound: one workgroup per (16 or 32 query rows, head); Q.K^T by
 // v_mfma_f32_16x16x32_f16 into an LDS score strip [rows][T], softmax in LDS, P.V by MFMA with V
@@ -144,6 +144,138 @@ __global__ __launch_bounds__(DEC_THREADS) void decode_attention_kernel(half_t* _
     for (int g = 0; g < DEC_GROUPS; ++g) o += gsum[g][tid];
     out[h * HD + tid] = round_f16(o);  // 529
   }
+}
+
+// ---- decode attention in two launches -----------------------------------------------------------
+// One compute unit's load path moves about 120 GB/s, so one workgroup per head cannot stream a
+// head's K and V (295 KB at T = 576, 1 MB at T = 2048) any faster than that, on 32 of 256 compute
+// units.  Split along T the scores need no cross-workgroup step at all, and the second launch
+// splits along the head's 128 output columns instead, each workgroup repeating the (cheap) softmax
+// of its head's row: no workgroup ever waits for another.
+//
+// dec_scores_kernel: workgroup (chunk of 64 cache rows, head): 16 lanes per row, 4 rows per
+//   thread group in flight; writes the fp16 scores of llama_cu.cu:400-428 to scores[head][t].
+// dec_softmax_pv_kernel: workgroup (32-column slice, head), 256 threads: requests its V slice
+//   first, then the reference's softmax over the row (the 256 threads are the reference's 256:
+//   same association of the sum, llama_cu.cu:433-499), then the weighted sum (511-531).
+constexpr int SC_ROWS = 64;      // cache rows per scores workgroup
+constexpr int PV_COLS = 32;      // output columns per second-stage workgroup
+constexpr int PV_FLIGHT = 16;    // 64-row passes whose loads are requested together (1024 rows)
+constexpr int SINGLE_LAUNCH_MAX_T = 1024;
+
+__global__ __launch_bounds__(256) void dec_scores_kernel(half_t* __restrict__ scores, const half_t* __restrict__ q,
+                                                         const half_t* __restrict__ k, int T_cap, int dim,
+                                                         const int* __restrict__ pos_dev) {
+  int T = T_cap;
+  if (pos_dev) T = min(max(*pos_dev + 1, 1), T_cap);
+  const int t0 = blockIdx.x * SC_ROWS;
+  if (t0 >= T) return;
+  const int h = blockIdx.y;
+  const int tid = threadIdx.x, sub = tid & 15, grp = tid >> 4;  // 16 row groups
+  const half8_t qh = *reinterpret_cast<const half8_t*>(q + h * HD + sub * 8);
+  const half_t* kh = k + h * HD + sub * 8;
+  half8_t kv[SC_ROWS / 16];
+#pragma unroll
+  for (int f = 0; f < SC_ROWS / 16; ++f) {
+    const int p = min(t0 + f * 16 + grp, T - 1);
+    kv[f] = __builtin_nontemporal_load(reinterpret_cast<const half8_t*>(kh + (size_t)p * dim));
+  }
+  const float denom = sqrtf((float)HD);
+#pragma unroll
+  for (int f = 0; f < SC_ROWS / 16; ++f) {
+    const int p = t0 + f * 16 + grp;
+    float s = 0.0f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) s = fmaf((float)qh[e], (float)kv[f][e], s);
+    s = row16_sum(s);
+    if (sub == 0 && p < T) scores[(size_t)h * T_cap + p] = round_f16(s / denom);  // 425
+  }
+}
+
+__global__ __launch_bounds__(256) void dec_softmax_pv_kernel(half_t* __restrict__ out,
+                                                             const half_t* __restrict__ scores,
+                                                             const half_t* __restrict__ v, int T_cap, int dim,
+                                                             const int* __restrict__ pos_dev) {
+  __shared__ half_t sc[MAX_T_DECODE];  // fp16 scores, then fp16 probabilities
+  __shared__ float gsum[64][PV_COLS + 1];
+  __shared__ float red[8];
+  int T = T_cap;
+  if (pos_dev) T = min(max(*pos_dev + 1, 1), T_cap);
+  const int slice = blockIdx.x, h = blockIdx.y;
+  const int tid = threadIdx.x, sub = tid & 3, grp = tid >> 2;  // 4 lanes x 16 bytes = the 32 columns of a row
+  const half_t* vh = v + h * HD + slice * PV_COLS + sub * 8;
+  // the first 1024 rows of the V slice: independent of everything below
+  half8_t vv[PV_FLIGHT];
+#pragma unroll
+  for (int f = 0; f < PV_FLIGHT; ++f) {
+    const int p = f * 64 + grp;
+    vv[f] = p < T ? __builtin_nontemporal_load(reinterpret_cast<const half8_t*>(vh + (size_t)p * dim)) : (half8_t)(0.0f);
+  }
+  for (int i = tid; i < T; i += 256) sc[i] = scores[(size_t)h * T_cap + i];
+  __syncthreads();
+  // softmax_rows: thread t owns elements t, t+256, ...
+  float m = -INFINITY;
+  for (int i = tid; i < T; i += 256) m = fmaxf(m, (float)sc[i]);
+  m = block256_max(m, red);
+  float s = 0.0f;
+  for (int i = tid; i < T; i += 256) s += expf((float)sc[i] - m);
+  const float total = block256_sum_ref_order(s, red);
+  for (int i = tid; i < T; i += 256) sc[i] = round_f16(expf((float)sc[i] - m) / total);  // 497
+  __syncthreads();
+  // matmul_qkv: row group g adds rows g, g+64, ... in ascending order, then the groups are added
+  float acc[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) acc[e] = 0.0f;
+  for (int p0 = 0; p0 < T; p0 += 64 * PV_FLIGHT) {
+    if (p0 > 0) {
+#pragma unroll
+      for (int f = 0; f < PV_FLIGHT; ++f) {
+        const int p = p0 + f * 64 + grp;
+        vv[f] = p < T ? __builtin_nontemporal_load(reinterpret_cast<const half8_t*>(vh + (size_t)p * dim))
+                      : (half8_t)(0.0f);
+      }
+    }
+#pragma unroll
+    for (int f = 0; f < PV_FLIGHT; ++f) {
+      const int p = p0 + f * 64 + grp;
+      if (p < T) {
+        const float prob = (float)sc[p];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc[e] = fmaf(prob, (float)vv[f][e], acc[e]);
+      }
+    }
+  }
+#pragma unroll
+  for (int e = 0; e < 8; ++e) gsum[grp][sub * 8 + e] = acc[e];
+  __syncthreads();
+  if (tid < PV_COLS) {
+    float o = 0.0f;
+#pragma unroll 8
+    for (int g = 0; g < 64; ++g) o += gsum[g][tid];
+    out[h * HD + slice * PV_COLS + tid] = round_f16(o);  // 529
+  }
+}
+
+// scores scratch: n_heads x T_cap halves of the per-device workspace
+int launch_decode_attention(half_t* out, const half_t* q, const half_t* k, const half_t* v, const int* pos_dev,
+                            int T_cap, int dim, int n_heads, hipStream_t s) {
+  device_state* st = current_device_state();
+  if (!st || !st->ready) return set_error(LCU_E_NOINIT, "lcu_attention: lcu_init has not run on this device");
+  LCU_REQUIRE((size_t)n_heads * T_cap * sizeof(half_t) <= st->workspace_bytes, "lcu_attention: workspace too small");
+  half_t* scores = (half_t*)st->workspace;
+  // up to 1024 cached rows the single launch wins (10.3 us against 11.0 us at T = 576: the second
+  // launch costs more than the spreading saves), beyond that the two launches do (21 us against
+  // 28 us at T = 2048)
+  if (T_cap <= SINGLE_LAUNCH_MAX_T) {
+    decode_attention_kernel<<<n_heads, DEC_THREADS, 0, s>>>(out, q, k, v, T_cap, dim, pos_dev);
+    LCU_LAUNCH_CHECK();
+    return LCU_OK;
+  }
+  dec_scores_kernel<<<dim3((T_cap + SC_ROWS - 1) / SC_ROWS, n_heads), 256, 0, s>>>(scores, q, k, T_cap, dim, pos_dev);
+  LCU_LAUNCH_CHECK();
+  dec_softmax_pv_kernel<<<dim3(HD / PV_COLS, n_heads), 256, 0, s>>>(out, scores, v, T_cap, dim, pos_dev);
+  LCU_LAUNCH_CHECK();
+  return LCU_OK;
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -352,10 +484,8 @@ int lcu_attention(void* out_dev, const void* q_dev, const void* k_dev, const voi
   hipStream_t s = as_stream(stream);
   if (n_new == 1) {
     LCU_REQUIRE(T <= MAX_T_DECODE, "lcu_attention: T %d exceeds %d", T, MAX_T_DECODE);
-    decode_attention_kernel<<<n_heads, DEC_THREADS, 0, s>>>((half_t*)out_dev, (const half_t*)q_dev,
-                                                            (const half_t*)k_dev, (const half_t*)v_dev, T, dim, nullptr);
-    LCU_LAUNCH_CHECK();
-    return LCU_OK;
+    return launch_decode_attention((half_t*)out_dev, (const half_t*)q_dev, (const half_t*)k_dev, (const half_t*)v_dev,
+                                   nullptr, T, dim, n_heads, s);
   }
   LCU_REQUIRE(T <= MAX_T_PREFILL, "lcu_attention: T %d exceeds %d for n_new > 1", T, MAX_T_PREFILL);
   // 16-row tiles when 32-row tiles would leave the grid under four workgroups per compute unit
@@ -396,11 +526,8 @@ int lcu_attention_decode(void* out_dev, const void* q_dev, const void* k_dev, co
               "lcu_attention_decode: dim %d / heads %d unsupported (head_dim must be 128, at most %d heads)", dim,
               n_heads, MAX_HEADS);
   LCU_REQUIRE(max_T > 0 && max_T <= MAX_T_DECODE, "lcu_attention_decode: max_T %d outside 1..%d", max_T, MAX_T_DECODE);
-  decode_attention_kernel<<<n_heads, DEC_THREADS, 0, as_stream(stream)>>>(
-      (half_t*)out_dev, (const half_t*)q_dev, (const half_t*)k_dev, (const half_t*)v_dev, max_T, dim,
-      (const int*)pos_dev);
-  LCU_LAUNCH_CHECK();
-  return LCU_OK;
+  return launch_decode_attention((half_t*)out_dev, (const half_t*)q_dev, (const half_t*)k_dev, (const half_t*)v_dev,
+                                 (const int*)pos_dev, max_T, dim, n_heads, as_stream(stream));
 }
 
 }  // extern "C"

@@ -314,7 +314,7 @@ void llama_context_impl::enqueue_layers(int n) {
       LCU_CHECK(lcu_decode_qkv(t_xq_.data(), kc, vc, t_norm_.data(), nullptr, L.wq.data.data(), L.wk.data.data(),
                                L.wv.data.data(), L.wq.scales.data(), L.wk.scales.data(), L.wv.scales.data(), block, dim,
                                heads, 0, t_step_.data(), p.norm_eps, rope_table_, context_len_, stream_));
-      LCU_CHECK(lcu_attention_decode(t_out_.data(), t_xq_.data(), kc, vc, t_step_.data(), context_len_, dim, heads,
+      LCU_CHECK(lcu_attention_decode(t_out_.data(), t_xq_.data(), kc, vc, t_step_.data(), decode_bound_, dim, heads,
                                      stream_));
     } else {
       char* k_new = kc + (size_t)sp * dim * 2;
@@ -395,6 +395,14 @@ short llama_context_impl::next_token(std::vector<short> const& new_tokens) {
   if (n == 1) {
     // A decode step is ~260 launches of a few microseconds each: the first one runs eagerly (and
     // loads the kernels), the second is captured into a HIP graph, every later one replays it.
+    // Decode attention has a form for short rows and one for long rows, chosen by the bound it is
+    // given; the graph is captured again when the position outgrows the short bound.
+    const int bound = (start_pos_ + 1 <= 1024 && context_len_ > 1024) ? 1024 : (int)context_len_;
+    if (decode_graph_ && bound != decode_bound_) {
+      LCU_CHECK(lcu_graph_destroy(decode_graph_));
+      decode_graph_ = nullptr;
+    }
+    decode_bound_ = bound;
     ++decode_calls_;
     if (!decode_graph_ && decode_calls_ >= 2) {
       LCU_CHECK(lcu_graph_begin_capture(stream_));

@@ -75,6 +75,7 @@ struct llama_context_impl final : public llama_context {
   } host_step_{};
   void* decode_graph_{nullptr};
   int decode_calls_{0};
+  int decode_bound_{0};  // the position bound the decode graph was captured with
   void* stream_{nullptr};
   void* rope_table_{nullptr};
   int last_n_{0};

@@ -109,6 +109,29 @@ def test_prefill_chunks_and_decode_agree(gpu):
     assert G.max_abs_rel(kb, ka) <= TOL and G.max_abs_rel(vb, va) <= TOL
 
 
+def test_decode_across_the_attention_form_boundary(gpu):
+    """Decode steps at positions 1020..1029: the first ones use the single-launch attention and a
+    graph captured with the bound 1024, the later ones the two-launch form and a new graph.  Every
+    step must agree with a fresh prefill of the same tokens."""
+    G = gpu
+    gm = G.P.Model(**SMALL, seed=4, weight_std=0.05)
+    toks = np.random.default_rng(2).integers(0, SMALL["n_vocab"], 1031).astype(np.int16)
+    a = G.P.Context(gm, context_len=2048, temperature=0.8)
+    a.next_token(toks[:1020])
+    b = G.P.Context(gm, context_len=2048, temperature=0.8)
+    for i in range(1020, 1030):
+        a.next_token(toks[i:i + 1])
+        b.clear_tokens()
+        b.next_token(toks[:i + 1])
+        assert G.max_abs_rel(a.logits(), b.logits()) <= TOL, i
+        assert G.max_abs_rel(a.hidden(1)[0], b.hidden(i + 1)[-1]) <= TOL, i
+    ka, va = a.kv(2, 1030)
+    kb, vb = b.kv(2, 1030)
+    assert G.max_abs_rel(ka, kb) <= TOL and G.max_abs_rel(va, vb) <= TOL
+    for o in (a, b, gm):
+        o.close()
+
+
 def test_context_api_behaviour(gpu):
     G = gpu
     gm = G.P.Model(**TINY, seed=1)

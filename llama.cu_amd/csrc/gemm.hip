@@ -356,25 +356,28 @@ __global__ __launch_bounds__(64 * WM * WN * KS, WM * WN * KS <= 4 ? 2 : 1) void 
   // two fp16 W tiles, then the code ring
   constexpr int A_STRIDE = U8 ? A_BYTES : A_BYTES + B_BYTES, B_STRIDE = U8 ? B_BYTES : A_BYTES + B_BYTES;
   constexpr int B_BASE = U8 ? NS * A_BYTES : A_BYTES, C_BASE = NS * A_BYTES + NB * B_BYTES;
+  constexpr int S_BYTES = THREADS * 4 * DC;  // scale ring slot: one dword per thread and chunk
+  constexpr int S_BASE = C_BASE + NS * C_BYTES;
+  constexpr int LDS_BYTES = NS * A_BYTES + NB * B_BYTES + (U8 ? NS * (C_BYTES + S_BYTES) : 0);
   constexpr int TM = BM / (32 * WM), TN = BN / (32 * WN);
   static_assert(PA >= 1 && PB >= 1 && DC >= 1 && NS >= 2 && NS <= 4, "unsupported configuration");
   static_assert(!U8 || NS == 3, "the uint8 schedule is written for a ring of three");
-  static_assert((PA + PB + DC) * (NS - 1) < 64, "vmcnt has 6 bits");
+  constexpr int P = PA + PB + (U8 ? DC : 0);  // requests per wavefront and batch
+  static_assert(P * (NS - 1) < 64, "vmcnt has 6 bits");
 
   extern __shared__ __attribute__((aligned(16))) unsigned char gemm_lds[];
 
   const int nb = tiles_m * tiles_n;
-  const int bid = blockIdx.x;
-  const int q = nb / NUM_XCD, r = nb % NUM_XCD;
-  const int xcd = bid % NUM_XCD, idx = bid / NUM_XCD;
-  const int logical = xcd * q + min(xcd, r) + idx;
-  const int tm = logical % tiles_m, tn = logical / tiles_m;
-  const int m0 = tm * BM, n0 = tn * BN;
-
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
   const int group = wave / NG, w4 = wave % NG;
   const int wm = (w4 % WM) * (BM / WM), wn = (w4 / WM) * (BN / WN);
+  // XCD-aware tile order, as in gemm_kernel
+  const int q = nb / NUM_XCD, r = nb % NUM_XCD;
+  const int xcd = blockIdx.x % NUM_XCD, idx = blockIdx.x / NUM_XCD;
+  const int logical = xcd * q + min(xcd, r) + idx;
+  const int tm = logical % tiles_m, tn = logical / tiles_m;
+  const int m0 = tm * BM, n0 = tn * BN;
 
   // loader: instruction j of this wavefront fills LDS bytes [(wave + j*NW) * 1024, +1024) of the
   // operand's region; lane l lands on tile row c / CR, chunk position c % CR, c = that index * 64 + l
@@ -397,29 +400,61 @@ __global__ __launch_bounds__(64 * WM * WN * KS, WM * WN * KS <= 4 ? 2 : 1) void 
   }
   const char* Ab = (const char*)A;
   const char* Wb = (const char*)W;
-  using gptr = const __attribute__((address_space(1))) void*;
-  using lptr = __attribute__((address_space(3))) void*;
+  // uint8: the chunks this thread dequantises (tile row, chunk in the row), their scale index at
+  // stage 0, and where the two fp16 chunks of a dequantised chunk go in the W tile
+  int d_scale[DC];
+  uint32_t d_src[DC], d_dst0[DC], d_dst1[DC];
+  const int nblk = U8 ? K / block : 0;
+  if constexpr (U8) {
+#pragma unroll
+    for (int i = 0; i < DC; ++i) {
+      const int c = tid + i * THREADS;
+      const int row = c / CPR, kc = c % CPR, f = (row / RPB) % CR;
+      d_scale[i] = min(n0 + row, N - 1) * nblk;
+      d_src[i] = (uint32_t)c * 16;
+      d_dst0[i] = (uint32_t)row * ROWB + (uint32_t)(((2 * kc) ^ f) * 16);
+      d_dst1[i] = (uint32_t)row * ROWB + (uint32_t)(((2 * kc + 1) ^ f) * 16);
+    }
+  }
+  // A request is written as inline assembly (M0 = LDS address of the wavefront's 1 KB, then the
+  // load), so that the compiler does not know about it: knowing, it treats the request like a FLAT
+  // access and waits for every LDS read in front of each matrix instruction.  Nothing else in this
+  // kernel uses M0.  The data lands in LDS, not in a register, so there is nothing here the
+  // compiler could copy too early; the waits for it (vmcnt) are the explicit ones below.
+  const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char*)gemm_lds;
+  auto request16 = [&](const void* g, uint32_t lds_off) {
+    const uint32_t m0 = __builtin_amdgcn_readfirstlane(lds0 + lds_off);
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(g), "s"(m0) : "memory");
+  };
+  auto request4 = [&](const void* g, uint32_t lds_off) {
+    const uint32_t m0 = __builtin_amdgcn_readfirstlane(lds0 + lds_off);
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %0, off" ::"v"(g), "s"(m0) : "memory");
+  };
   const int nt = K / BKS;
-  // load instruction `idx` (0 .. PA+PB-1) of this wavefront for batch `stage` into ring slot `slot`:
-  // the lhs tile of that stage, and the W tile of that stage (fp16) or the codes of the stage after
-  // it (uint8; past the end the last stage is fetched again and never used)
+  // request `idx` (0 .. P-1) of this wavefront for batch `stage` into ring slot `slot`: the lhs tile
+  // of that stage, and the W tile of that stage (fp16) or the codes and scales of the stage after it
+  // (uint8; past the end the last stage is fetched again and never used)
   auto issue_one = [&](int stage, int slot, int idx) {
     if (idx < PA) {
-      unsigned char* dst = gemm_lds + slot * A_STRIDE + (wave + idx * NW) * 1024;
-      __builtin_amdgcn_global_load_lds((gptr)(Ab + (size_t)stage * (BKS * 2) + a_off[idx]), (lptr)dst, 16, 0, 0);
+      request16(Ab + (size_t)stage * (BKS * 2) + a_off[idx], slot * A_STRIDE + (wave + idx * NW) * 1024);
     } else if constexpr (U8) {
       const int cslot = slot + 1 == NS ? 0 : slot + 1;
-      unsigned char* dst = gemm_lds + C_BASE + cslot * C_BYTES + (wave + (idx - PA) * NW) * 1024;
-      __builtin_amdgcn_global_load_lds((gptr)(Wb + (size_t)min(stage + 1, nt - 1) * BKS + b_off[idx - PA]), (lptr)dst, 16,
-                                       0, 0);
+      const int st1 = min(stage + 1, nt - 1);
+      if (idx < PA + PB) {
+        request16(Wb + (size_t)st1 * BKS + b_off[idx - PA], C_BASE + cslot * C_BYTES + (wave + (idx - PA) * NW) * 1024);
+      } else {
+        const int i = idx - PA - PB;  // the dword that holds this thread's fp16 scale of chunk i
+        const int kc = (tid + i * THREADS) % CPR;
+        const int at = d_scale[i] + (st1 * BKS + kc * 16) / block;
+        request4(S + (at & ~1), S_BASE + cslot * S_BYTES + (i * NW + wave) * 256);
+      }
     } else {
-      unsigned char* dst = gemm_lds + B_BASE + slot * B_STRIDE + (wave + (idx - PA) * NW) * 1024;
-      __builtin_amdgcn_global_load_lds((gptr)(Wb + (size_t)stage * (BKS * 2) + b_off[idx - PA]), (lptr)dst, 16, 0, 0);
+      request16(Wb + (size_t)stage * (BKS * 2) + b_off[idx - PA], B_BASE + slot * B_STRIDE + (wave + (idx - PA) * NW) * 1024);
     }
   };
   auto issue = [&](int stage, int slot) {
 #pragma unroll
-    for (int idx = 0; idx < PA + PB; ++idx) issue_one(stage, slot, idx);
+    for (int idx = 0; idx < P; ++idx) issue_one(stage, slot, idx);
   };
 
   float16_t acc[TM][TN];
@@ -441,37 +476,16 @@ __global__ __launch_bounds__(64 * WM * WN * KS, WM * WN * KS <= 4 ? 2 : 1) void 
   for (int s4 = 0; s4 < BK / 16; ++s4) pos[s4] = (uint32_t)(((gbase + 2 * s4) ^ fr) * 16);
   const uint32_t a_row = (uint32_t)(wm + frag_row) * ROWB, b_row = (uint32_t)B_BASE + (uint32_t)(wn + frag_row) * ROWB;
 
-  // uint8: the chunks this thread dequantises (tile row, chunk in the row), their scale index at
-  // stage 0, and where the two fp16 chunks of a dequantised chunk go in the W tile
-  int d_scale[DC];
-  uint32_t d_src[DC], d_dst0[DC], d_dst1[DC];
-  half_t sc_cur[DC], sc_nxt[DC];
-  const int nblk = U8 ? K / block : 0;
-  if constexpr (U8) {
-#pragma unroll
-    for (int i = 0; i < DC; ++i) {
-      const int c = tid + i * THREADS;
-      const int row = c / CPR, kc = c % CPR, f = (row / RPB) % CR;
-      d_scale[i] = min(n0 + row, N - 1) * nblk;
-      d_src[i] = (uint32_t)c * 16;
-      d_dst0[i] = (uint32_t)row * ROWB + (uint32_t)(((2 * kc) ^ f) * 16);
-      d_dst1[i] = (uint32_t)row * ROWB + (uint32_t)(((2 * kc + 1) ^ f) * 16);
-    }
-  }
-  auto load_scales = [&](half_t (&sc)[DC], int stage) {
-    const int st = min(stage, nt - 1);
-#pragma unroll
-    for (int i = 0; i < DC; ++i) {
-      const int kc = (tid + i * THREADS) % CPR;
-      sc[i] = S[d_scale[i] + (st * BKS + kc * 16) / block];
-    }
-  };
-  // codes in ring slot `cslot` -> fp16 W tile `bslot`
-  auto dequantise = [&](int cslot, int bslot, const half_t (&sc)[DC]) {
+  // codes and scales in ring slot `cslot` (they belong to K stage `stage`) -> fp16 W tile `bslot`
+  auto dequantise = [&](int cslot, int bslot, int stage) {
 #pragma unroll
     for (int i = 0; i < DC; ++i) {
       const uint4_t q = *reinterpret_cast<const uint4_t*>(gemm_lds + C_BASE + cslot * C_BYTES + d_src[i]);
-      const half_t s2 = sc[i] * (half_t)2.0f;
+      const uint32_t pair = *reinterpret_cast<const uint32_t*>(gemm_lds + S_BASE + cslot * S_BYTES + i * THREADS * 4 + tid * 4);
+      const int kc = (tid + i * THREADS) % CPR;
+      const int at = d_scale[i] + (stage * BKS + kc * 16) / block;  // the request fetched the dword at (at & ~1)
+      const half_t sc = __builtin_bit_cast(half_t, (uint16_t)((at & 1) ? pair >> 16 : pair & 0xffffu));
+      const half_t s2 = sc * (half_t)2.0f;
       const half2_t s2v = {s2, s2};
       half2_t d[8];
 #pragma unroll
@@ -487,41 +501,25 @@ __global__ __launch_bounds__(64 * WM * WN * KS, WM * WN * KS <= 4 ? 2 : 1) void 
     }
   };
 
-  // ---- the stage loop, scheduled by hand ------------------------------------------------------
-  // The LDS reads and their waits are written as inline assembly: with global_load_lds requests
-  // outstanding the compiler waits for *every* LDS read in front of each matrix instruction group
-  // (it models the requests like FLAT accesses), which exposes the LDS latency four times per
-  // stage.  Here a group waits only for its own fragments (lgkmcnt counts LDS reads in order;
-  // the global_load_lds requests count in vmcnt), and the synchronisation for the next stage
-  // sits in front of the last group, so the first fragments of the next stage are already on
-  // their way while that group runs and the matrix core never drains at a stage boundary.
-  //
+  // ---- the stage loop --------------------------------------------------------------------------
   // K slice s of a stage uses fragment buffer s & 1.  Per stage and wavefront:
-  //   slices 0..2: read slice s+1 | wait for slice s | request a third of the stage NS-1 ahead | multiply s
-  //   slice 3:     wait for slice 3 (nothing else is pending: this wavefront is done reading the
-  //                stage) | wait for the own requests of the next stage | barrier | read slice 0 of
-  //                the next stage | multiply 3
-  constexpr int S4 = BK / 16, P = PA + PB;
+  //   slices 0..2: read slice s+1 | request a third of the batch NS-1 ahead | multiply slice s
+  //   slice 3:     wait for this wavefront's LDS accesses (it is then done with the stage) | wait
+  //                for its own requests of the next stage | barrier | read slice 0 of the next
+  //                stage | multiply slice 3
+  // so fragments are always requested one slice before the matrix instructions that use them, also
+  // across the stage boundary.  The fragment reads are ordinary loads: the compiler counts them
+  // (lgkmcnt) and waits for exactly the fragments an instruction needs.
+  constexpr int S4 = BK / 16;
   static_assert(S4 == 4, "the schedule below is written for four K slices per stage");
-  const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char*)gemm_lds;
   half8_t fa[2][TM], fb[2][TN];
   auto read_frags = [&](int buf, int slot, int bslot, int s4) {
-    const uint32_t pa = lds0 + slot * A_STRIDE + a_row + pos[s4], pb = lds0 + bslot * B_STRIDE + b_row + pos[s4];
+    const unsigned char* pa = gemm_lds + slot * A_STRIDE + a_row + pos[s4];
+    const unsigned char* pb = gemm_lds + bslot * B_STRIDE + b_row + pos[s4];
 #pragma unroll
-    for (int i = 0; i < TM; ++i) {
-      asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(fa[buf][i]) : "v"(pa), "n"(i * 32 * ROWB));
-    }
+    for (int i = 0; i < TM; ++i) fa[buf][i] = *reinterpret_cast<const half8_t*>(pa + i * 32 * ROWB);
 #pragma unroll
-    for (int j = 0; j < TN; ++j) {
-      asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(fb[buf][j]) : "v"(pb), "n"(j * 32 * ROWB));
-    }
-  };
-  // the fragments of `buf` become usable only after the wait: redefine them behind it
-  auto frags_ready = [&](int buf) {
-#pragma unroll
-    for (int i = 0; i < TM; ++i) asm volatile("" : "+v"(fa[buf][i]));
-#pragma unroll
-    for (int j = 0; j < TN; ++j) asm volatile("" : "+v"(fb[buf][j]));
+    for (int j = 0; j < TN; ++j) fb[buf][j] = *reinterpret_cast<const half8_t*>(pb + j * 32 * ROWB);
   };
   auto multiply = [&](int buf) {
 #pragma unroll
@@ -534,49 +532,44 @@ __global__ __launch_bounds__(64 * WM * WN * KS, WM * WN * KS <= 4 ? 2 : 1) void 
   };
   // one stage (lhs in ring slot `slot`, W tile `bslot`); FETCH: request batch `next` into slot
   // `fill`; MORE: another stage follows (slots `nslot`, `nbslot`), whose own requests are complete
-  // once at most PEND younger ones are outstanding.  uint8 with MORE: the scales of the stage after
-  // the next are requested first, and between the first two slices the codes of the next stage
-  // (ring slot nslot) become its fp16 tile nbslot.  Those LDS accesses are the compiler's; being
-  // younger than the fragments a slice waits for, they can only make the hand-counted waits stricter.
+  // once at most PEND younger ones are outstanding.  uint8 with MORE: between the first two slices
+  // the codes of the next stage (ring slot nslot) become its fp16 tile nbslot.
   auto stage = [&](int slot, int bslot, auto fetch, int next, int fill, auto more, auto pend, int nslot, int nbslot,
                    int t) {
     constexpr bool FETCH = decltype(fetch)::value, MORE = decltype(more)::value;
     constexpr int PEND = decltype(pend)::value;
-    if constexpr (U8 && MORE) load_scales(sc_nxt, t + 2);
 #pragma unroll
     for (int s4 = 0; s4 < 3; ++s4) {
       read_frags((s4 + 1) & 1, slot, bslot, s4 + 1);
-      asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(TM + TN) : "memory");
-      frags_ready(s4 & 1);
       if constexpr (FETCH) {
 #pragma unroll
         for (int idx = s4 * P / 3; idx < (s4 + 1) * P / 3; ++idx) issue_one(next, fill, idx);
       }
+      __builtin_amdgcn_sched_barrier(0);
       multiply(s4 & 1);
+      __builtin_amdgcn_sched_barrier(0);
       if constexpr (U8 && MORE) {
-        if (s4 == 0) dequantise(nslot, nbslot, sc_cur);
+        if (s4 == 0) {
+          dequantise(nslot, nbslot, t + 1);
+          __builtin_amdgcn_sched_barrier(0);
+        }
       }
     }
-    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-    frags_ready(1);
     if constexpr (MORE) {
+      // this wavefront's reads of the stage (and its writes of the next fp16 tile) are complete
+      // before it lets the others overwrite the slot / read the tile
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
       wait_vmcnt<PEND>();
       asm volatile("s_barrier" ::: "memory");
       read_frags(0, nslot, nbslot, 0);
+      __builtin_amdgcn_sched_barrier(0);
     }
     multiply(1);
-    if constexpr (U8 && MORE) {
-#pragma unroll
-      for (int i = 0; i < DC; ++i) sc_cur[i] = sc_nxt[i];
-    }
+    __builtin_amdgcn_sched_barrier(0);
   };
 
-  constexpr int PS = U8 ? P + DC : P;  // vector-memory requests per stage: the batch, and the scale loads
   if constexpr (U8) {
-    // scales of stages 0 and 1, codes of stage 0 (into code slot 0), then the first batches
-    half_t sc0[DC];
-    load_scales(sc0, 0);
-    load_scales(sc_cur, 1);
+    // codes and scales of stage 0 (batch -1, into slot 0 of their rings), then the first batches
 #pragma unroll
     for (int idx = PA; idx < P; ++idx) issue_one(-1, NS - 1, idx);
 #pragma unroll
@@ -584,12 +577,12 @@ __global__ __launch_bounds__(64 * WM * WN * KS, WM * WN * KS <= 4 ? 2 : 1) void 
       if (s0 < nt) issue(s0, s0);
     }
     if (nt > 1) {
-      wait_vmcnt<(NS - 1) * P>();  // everything older than the batches: the codes of stage 0
+      wait_vmcnt<(NS - 1) * P>();  // everything older than the batches: codes and scales of stage 0
     } else {
       wait_vmcnt<0>();
     }
     asm volatile("s_barrier" ::: "memory");
-    dequantise(0, 0, sc0);
+    dequantise(0, 0, 0);
   } else {
 #pragma unroll
     for (int s0 = 0; s0 < NS - 1; ++s0) {
@@ -608,10 +601,10 @@ __global__ __launch_bounds__(64 * WM * WN * KS, WM * WN * KS <= 4 ? 2 : 1) void 
   auto next_of = [](int v) { return v + 1 == NS ? 0 : v + 1; };
   const int n_main = max(nt - (NS - 1), 0);
   for (int t = 0; t < n_main; ++t) {
-    // after this stage's requests (batch t+NS-1 and, uint8, scale loads), stages t+2 .. t+NS-1 may
-    // stay in flight when stage t+1 must have landed
+    // after this stage's requests (batch t+NS-1), batches t+2 .. t+NS-1 may stay in flight when
+    // batch t+1 must have landed
     stage(slot, U8 ? (t & 1) : slot, std::true_type{}, t + NS - 1, fill, std::true_type{},
-          std::integral_constant<int, (NS - 2) * PS>{}, next_of(slot), U8 ? ((t + 1) & 1) : next_of(slot), t);
+          std::integral_constant<int, (NS - 2) * P>{}, next_of(slot), U8 ? ((t + 1) & 1) : next_of(slot), t);
     slot = next_of(slot);
     fill = next_of(fill);
   }
@@ -643,35 +636,38 @@ __global__ __launch_bounds__(64 * WM * WN * KS, WM * WN * KS <= 4 ? 2 : 1) void 
       }
     }
     __syncthreads();
-    if (group == 1) return;
+    if (group == 0) {
 #pragma unroll
-    for (int i = 0; i < TM; ++i) {
+      for (int i = 0; i < TM; ++i) {
 #pragma unroll
-      for (int j = 0; j < TN; ++j) {
+        for (int j = 0; j < TN; ++j) {
 #pragma unroll
-        for (int v = 0; v < 16; ++v) {
-          acc[i][j][v] += part[(((w4 * TM + i) * TN + j) * 16 + v) * 64 + lane];
+          for (int v = 0; v < 16; ++v) {
+            acc[i][j][v] += part[(((w4 * TM + i) * TN + j) * 16 + v) * 64 + lane];
+          }
         }
       }
     }
   }
 
   // epilogue as in gemm_kernel (llama_cu.cu:208-215)
+  if (group == 0) {
 #pragma unroll
-  for (int i = 0; i < TM; ++i) {
+    for (int i = 0; i < TM; ++i) {
 #pragma unroll
-    for (int j = 0; j < TN; ++j) {
-      const int gn = n0 + wn + j * 32 + (lane & 31);
+      for (int j = 0; j < TN; ++j) {
+        const int gn = n0 + wn + j * 32 + (lane & 31);
 #pragma unroll
-      for (int v = 0; v < 16; ++v) {
-        const int gm = m0 + wm + i * 32 + (v >> 2) * 8 + (lane >> 5) * 4 + (v & 3);
-        if (gm < M && gn < N) {
-          half_t* p = out + (size_t)gm * N + gn;
-          float val = acc[i][j][v];
-          if (beta != 0.0f) {
-            val = fmaf(beta, (float)*p, val);
+        for (int v = 0; v < 16; ++v) {
+          const int gm = m0 + wm + i * 32 + (v >> 2) * 8 + (lane >> 5) * 4 + (v & 3);
+          if (gm < M && gn < N) {
+            half_t* p = out + (size_t)gm * N + gn;
+            float val = acc[i][j][v];
+            if (beta != 0.0f) {
+              val = fmaf(beta, (float)*p, val);
+            }
+            *p = round_f16(val);
           }
-          *p = round_f16(val);
         }
       }
     }
@@ -682,7 +678,9 @@ template <int BM, int BN, int WM, int WN, int KS, int NS, bool U8>
 int launch_dl(half_t* out, const half_t* A, const void* W, const half_t* S, int M, int K, int N, int block,
               float beta, hipStream_t st) {
   constexpr int ROWB = BK * KS * 2;
-  constexpr size_t lds = (size_t)NS * BM * ROWB + (size_t)(U8 ? 2 : NS) * BN * ROWB + (U8 ? (size_t)NS * BN * BK * KS : 0);
+  constexpr int DCH = U8 ? BN * (BK * KS / 16) / (64 * WM * WN * KS) : 0;  // scale dwords per thread and stage
+  constexpr size_t lds = (size_t)NS * BM * ROWB + (size_t)(U8 ? 2 : NS) * BN * ROWB +
+                         (U8 ? (size_t)NS * (BN * BK * KS + 64 * WM * WN * KS * 4 * DCH) : 0);
   static_assert(lds <= 160 * 1024, "rings do not fit LDS");
   static_assert(KS == 1 || lds >= (size_t)BM * BN * 4 / 2, "LDS must hold one group's accumulators");
   const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;

@@ -149,10 +149,11 @@ def test_gemv_u8_dequant_is_exact(gpu):
 
 # the shapes cover every tile configuration of the dispatcher: 128x64 with two wavefront groups,
 # 256x128, 128x128 with eight wavefronts (160..255 tiles: N = 5120), 128x64 with two workgroups per
-# compute unit (N = 4160), 128x128 with four wavefronts (M = 1024, N = 4096), and ragged K / M / N
+# compute unit (N = 4160), 128x128 with four wavefronts (M = 1024, N = 4096), ragged K / M / N, and
+# grids with more tiles than the chip holds workgroups at once (the last three)
 @pytest.mark.parametrize("M,K,N", [(512, 4096, 4096), (512, 4096, 11008), (512, 11008, 4096), (128, 256, 128),
                                    (7, 64, 24), (130, 200, 70), (33, 1024, 257), (512, 256, 5120), (512, 384, 4160),
-                                   (1024, 256, 4096), (500, 128, 5100)])
+                                   (1024, 256, 4096), (500, 128, 5100), (4096, 128, 4096), (512, 256, 17920), (2100, 128, 8200)])
 def test_gemm_f16(gpu, M, K, N):
     G = gpu
     x = normal((M, K), 0, 300, 1.0)
@@ -184,7 +185,7 @@ def test_gemm_exact_cases(gpu):
 
 @pytest.mark.parametrize("M,K,N", [(512, 4096, 4096), (512, 4096, 11008), (512, 11008, 4096), (16, 256, 128),
                                    (130, 384, 70), (512, 256, 5120), (512, 384, 4160), (1024, 256, 4096),
-                                   (500, 128, 5100), (40, 384, 300)])
+                                   (500, 128, 5100), (40, 384, 300), (4096, 128, 4096), (512, 256, 17920)])
 def test_gemm_u8(gpu, M, K, N):
     G = gpu
     x = normal((M, K), 0, 400, 1.0)

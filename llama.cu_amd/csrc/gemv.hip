@@ -10,9 +10,10 @@
 //     before anything else happens in the workgroup (before x is staged or normalised), and the
 //     next batch is requested before the current one is consumed
 //   - each lane loads the pieces of x (or of the norm weights) that match its weights along with
-//     them; when x must be RMS-normalised first, every workgroup stages x in LDS with two 16-byte
-//     loads per thread, reduces the sum of squares there and normalises its pieces in registers
-//     (global load instructions per workgroup are what this prologue must keep few)
+//     them; when x must be RMS-normalised first, every workgroup requests x before its weights
+//     (loads return in request order), stages it in LDS, reduces the sum of squares there while
+//     the weights are on their way and normalises its pieces in registers (global load
+//     instructions per workgroup are what this prologue must keep few)
 //   - products accumulate in fp32 per lane, lanes combine with xor shuffles, wavefronts through
 //     LDS, thread 0 applies the epilogue (residual add, RoPE, SiLU*mul) and rounds once to fp16
 // uint8 weights are dequantised in packed fp16 to bit-for-bit fp16((q - 127.5) * scale), the value
@@ -21,6 +22,8 @@
 // the dequantisation arithmetic, not HBM, is what bounds this kernel on large matrices.
 #include "common.hpp"
 
+#include <type_traits>
+
 using namespace lcu;
 
 namespace {
@@ -28,25 +31,51 @@ namespace {
 constexpr int GEMV_THREADS = 256;
 constexpr int GEMV_WAVES = GEMV_THREADS / WAVE;
 
-// x is copied to LDS with 16-byte loads; the sum of squares is then taken from LDS in the
-// reference's order (llama_cu.cu:75-100: thread t owns elements t, t+256, ...;
-// block256_sum_ref_order), then 1/sqrt(mean + eps) with IEEE operations.  Few global load
-// instructions matter here: every workgroup of a kernel repeats this.  Every thread returns the
-// same value; xs holds the raw x afterwards.
-__device__ __forceinline__ float stage_x_rms_inv(half_t* xs, const half_t* __restrict__ x, int K, float eps,
-                                                 float* red) {
-  for (int i = threadIdx.x * 8; i < K; i += GEMV_THREADS * 8) {
-    *reinterpret_cast<uint4*>(xs + i) = *reinterpret_cast<const uint4*>(x + i);
-  }
-  __syncthreads();
-  float s = 0.0f;
-  for (int i = threadIdx.x; i < K; i += GEMV_THREADS) {
-    const float v = (float)xs[i];
-    s = fmaf(v, v, s);
-  }
-  const float total = block256_sum_ref_order(s, red);
-  return 1.0f / sqrtf(total / (float)K + eps);
+// RMS statistics of x inside a GEMV workgroup.  Loads come back in the order they were requested,
+// so the pieces of x are requested first (load), before the workgroup's weights: the norm is then
+// worked out while the weights are still on their way instead of after them.  reduce() copies x to
+// LDS and takes the sum of squares from there in the reference's order (llama_cu.cu:75-100: thread
+// t owns elements t, t+256, ...; block256_sum_ref_order), then 1/sqrt(mean + eps) with IEEE
+// operations.  Every thread returns the same value; xs holds the raw x afterwards.  XN 16-byte
+// pieces per thread cover K <= 2048 * XN; xs holds 2048 * XN halves.
+// keeps the memory requests written above it above the ones written below it
+__device__ __forceinline__ void issue_order_fence() {
+  __builtin_amdgcn_sched_barrier(0);
+  asm volatile("" ::: "memory");
+  __builtin_amdgcn_sched_barrier(0);
 }
+
+template <int XN>
+struct x_stage_t {
+  uint4_t v[XN > 0 ? XN : 1];
+  __device__ __forceinline__ void load(const half_t* x, int K) {
+    // the pointer passes through an empty asm so that these loads are ordinary ones to the
+    // compiler: loads from a const __restrict__ kernel argument may cross issue_order_fence()
+    asm volatile("" : "+s"(x));
+    typedef const __attribute__((address_space(1))) uint4_t* global_ptr_t;
+#pragma unroll
+    for (int j = 0; j < XN; ++j) {
+      const int i = min((int)(threadIdx.x + j * GEMV_THREADS) * 8, K - 8);
+      v[j] = *(global_ptr_t)(x + i);
+    }
+  }
+  __device__ __forceinline__ float reduce(half_t* xs, int K, float eps, float* red) const {
+#pragma unroll
+    for (int j = 0; j < XN; ++j) {
+      // unconditional (xs holds 2048 * XN halves): a conditional store lets the compiler move the
+      // load down to it, behind the weights
+      *reinterpret_cast<uint4_t*>(xs + (threadIdx.x + j * GEMV_THREADS) * 8) = v[j];
+    }
+    __syncthreads();
+    float s = 0.0f;
+    for (int i = threadIdx.x; i < K; i += GEMV_THREADS) {
+      const float e = (float)xs[i];
+      s = fmaf(e, e, s);
+    }
+    const float total = block256_sum_ref_order(s, red);
+    return 1.0f / sqrtf(total / (float)K + eps);
+  }
+};
 
 // rms_norm applied to 8 elements in registers: fp16(w * fp16(x * rms_inv)), llama_cu.cu:103-106
 __device__ __forceinline__ half8_t normed(half8_t x, half8_t w, float rms_inv) {
@@ -338,25 +367,33 @@ struct ffn_up_tasks {
 
 // ---- kernels -------------------------------------------------------------------------------------
 // one workgroup per task (blockIdx.x)
-template <bool U8, int R, int U, bool NORM>
+// XN > 0: x is RMS-normalised first, from XN 16-byte pieces per thread (x_stage_t)
+template <bool U8, int R, int U, int XN>
 __global__ __launch_bounds__(GEMV_THREADS) void gemv_kernel(half_t* __restrict__ out, const half_t* __restrict__ x,
                                                             const half_t* __restrict__ norm_w, const void* __restrict__ W,
                                                             const half_t* __restrict__ S, int K, int N, int block,
                                                             float beta, float eps) {
-  extern __shared__ half_t xs[];  // K halves when NORM, else unused
+  extern __shared__ half_t xs[];  // 2048 * XN halves
   __shared__ float red[8];
   __shared__ float part[GEMV_WAVES * R];
+  constexpr bool NORM = XN > 0;
   plain_tasks<U8, R> tk{W, S, out, K, N, U8 ? K / block : 0, beta};
   stream_t<U8, R, U, NORM, plain_tasks<U8, R>> st(tk, x, norm_w, K, block, blockIdx.x);
-  st.begin();
   float rms_inv = 1.0f;
   if constexpr (NORM) {
-    rms_inv = stage_x_rms_inv(xs, x, K, eps, red);
+    x_stage_t<XN> xp;
+    xp.load(x, K);
+    issue_order_fence();
+    st.begin();
+    issue_order_fence();
+    rms_inv = xp.reduce(xs, K, eps, red);
+  } else {
+    st.begin();
   }
   st.run(xs, rms_inv, part);
 }
 
-template <bool U8, int U, bool NORM>
+template <bool U8, int U, int XN>
 __global__ __launch_bounds__(GEMV_THREADS) void decode_qkv_kernel(
     half_t* __restrict__ q_out, half_t* __restrict__ k_row, half_t* __restrict__ v_row, const half_t* __restrict__ x,
     const half_t* __restrict__ norm_w, const void* __restrict__ wq, const void* __restrict__ wk,
@@ -380,16 +417,23 @@ __global__ __launch_bounds__(GEMV_THREADS) void decode_qkv_kernel(
   const half_t* S = which == 0 ? sq : (which == 1 ? sk : sv);
   half_t* dst = which == 0 ? q_out : (which == 1 ? k_row : v_row);
   qkv_tasks<U8> tk{W, S, dst, which == 2 ? nullptr : rope_row, dim, head_dim, U8 ? dim / block : 0, which * half_dim};
+  constexpr bool NORM = XN > 0;
   stream_t<U8, 2, U, NORM, qkv_tasks<U8>> st(tk, x, norm_w, dim, block, blockIdx.x);
-  st.begin();
   float rms_inv = 1.0f;
   if constexpr (NORM) {
-    rms_inv = stage_x_rms_inv(xs, x, dim, eps, red);
+    x_stage_t<XN> xp;
+    xp.load(x, dim);
+    issue_order_fence();
+    st.begin();
+    issue_order_fence();
+    rms_inv = xp.reduce(xs, dim, eps, red);
+  } else {
+    st.begin();
   }
   st.run(xs, rms_inv, part);
 }
 
-template <bool U8, int U, bool NORM>
+template <bool U8, int U, int XN>
 __global__ __launch_bounds__(GEMV_THREADS) void decode_ffn_up_kernel(
     half_t* __restrict__ out, const half_t* __restrict__ x, const half_t* __restrict__ norm_w,
     const void* __restrict__ w1, const void* __restrict__ w3, const half_t* __restrict__ s1,
@@ -398,13 +442,32 @@ __global__ __launch_bounds__(GEMV_THREADS) void decode_ffn_up_kernel(
   __shared__ float red[8];
   __shared__ float part[GEMV_WAVES * 2];
   ffn_up_tasks<U8> tk{w1, w3, s1, s3, out, dim, U8 ? dim / block : 0};
+  constexpr bool NORM = XN > 0;
   stream_t<U8, 2, U, NORM, ffn_up_tasks<U8>> st(tk, x, norm_w, dim, block, blockIdx.x);
-  st.begin();
   float rms_inv = 1.0f;
   if constexpr (NORM) {
-    rms_inv = stage_x_rms_inv(xs, x, dim, eps, red);
+    x_stage_t<XN> xp;
+    xp.load(x, dim);
+    issue_order_fence();
+    st.begin();
+    issue_order_fence();
+    rms_inv = xp.reduce(xs, dim, eps, red);
+  } else {
+    st.begin();
   }
   st.run(xs, rms_inv, part);
+}
+
+// calls f with the number of 16-byte pieces of x per thread (x_stage_t) that covers dim <= 24576
+template <class F>
+void with_x_pieces(int dim, F&& f) {
+  if (dim <= 4096) {
+    f(std::integral_constant<int, 2>{});
+  } else if (dim <= 8192) {
+    f(std::integral_constant<int, 4>{});
+  } else {
+    f(std::integral_constant<int, 12>{});
+  }
 }
 
 int check_quant_args(const char* who, const void* scales, int K, int block) {
@@ -421,9 +484,9 @@ namespace lcu {
 // M == 1 paths of lcu_gemm_f16_nt / lcu_gemm_f16u8_nt
 int gemv_f16(half_t* out, const half_t* x, const half_t* W, int K, int N, float beta, hipStream_t st) {
   if (K > 4096) {
-    gemv_kernel<false, 2, 2, false><<<(N + 1) / 2, GEMV_THREADS, 0, st>>>(out, x, nullptr, W, nullptr, K, N, 0, beta, 0.f);
+    gemv_kernel<false, 2, 2, 0><<<(N + 1) / 2, GEMV_THREADS, 0, st>>>(out, x, nullptr, W, nullptr, K, N, 0, beta, 0.f);
   } else {
-    gemv_kernel<false, 1, 2, false><<<N, GEMV_THREADS, 0, st>>>(out, x, nullptr, W, nullptr, K, N, 0, beta, 0.f);
+    gemv_kernel<false, 1, 2, 0><<<N, GEMV_THREADS, 0, st>>>(out, x, nullptr, W, nullptr, K, N, 0, beta, 0.f);
   }
   LCU_LAUNCH_CHECK();
   return LCU_OK;
@@ -432,9 +495,9 @@ int gemv_f16(half_t* out, const half_t* x, const half_t* W, int K, int N, float 
 int gemv_u8(half_t* out, const half_t* x, const uint8_t* W, const half_t* S, int K, int N, int block, float beta,
             hipStream_t st) {
   if (N >= 8192) {
-    gemv_kernel<true, 4, 1, false><<<(N + 3) / 4, GEMV_THREADS, 0, st>>>(out, x, nullptr, W, S, K, N, block, beta, 0.f);
+    gemv_kernel<true, 4, 1, 0><<<(N + 3) / 4, GEMV_THREADS, 0, st>>>(out, x, nullptr, W, S, K, N, block, beta, 0.f);
   } else {
-    gemv_kernel<true, 2, 1, false><<<(N + 1) / 2, GEMV_THREADS, 0, st>>>(out, x, nullptr, W, S, K, N, block, beta, 0.f);
+    gemv_kernel<true, 2, 1, 0><<<(N + 1) / 2, GEMV_THREADS, 0, st>>>(out, x, nullptr, W, S, K, N, block, beta, 0.f);
   }
   LCU_LAUNCH_CHECK();
   return LCU_OK;
@@ -465,30 +528,33 @@ int lcu_decode_qkv(void* q_out_dev, void* k_cache_dev, void* v_cache_dev, const 
   half_t* v_row = (half_t*)v_cache_dev + (size_t)pos * dim;
   const float2* rope_row = (const float2*)rope_table_dev + (size_t)pos * (head_dim / 2);
   const int grid = 3 * dim / 2;
-  const size_t lds = (size_t)dim * 2;
   hipStream_t st = as_stream(stream);
   if (block > 0) {
     int rc = check_quant_args("lcu_decode_qkv", sq_dev, dim, block);
     if (rc) return rc;
     LCU_REQUIRE(sk_dev && sv_dev, "lcu_decode_qkv: quantised weights need scales");
     if (norm_w_dev) {
-      decode_qkv_kernel<true, 1, true><<<grid, GEMV_THREADS, lds, st>>>(
-          (half_t*)q_out_dev, k_row, v_row, (const half_t*)x_dev, (const half_t*)norm_w_dev, wq_dev, wk_dev, wv_dev,
-          (const half_t*)sq_dev, (const half_t*)sk_dev, (const half_t*)sv_dev, block, dim, head_dim, eps, rope_row, (const int*)pos_dev,
-          table_positions - 1);
+      with_x_pieces(dim, [&](auto xn) {
+        decode_qkv_kernel<true, 1, decltype(xn)::value><<<grid, GEMV_THREADS, decltype(xn)::value * 4096, st>>>(
+            (half_t*)q_out_dev, k_row, v_row, (const half_t*)x_dev, (const half_t*)norm_w_dev, wq_dev, wk_dev, wv_dev,
+            (const half_t*)sq_dev, (const half_t*)sk_dev, (const half_t*)sv_dev, block, dim, head_dim, eps, rope_row,
+            (const int*)pos_dev, table_positions - 1);
+      });
     } else {
-      decode_qkv_kernel<true, 1, false><<<grid, GEMV_THREADS, 0, st>>>(
+      decode_qkv_kernel<true, 1, 0><<<grid, GEMV_THREADS, 0, st>>>(
           (half_t*)q_out_dev, k_row, v_row, (const half_t*)x_dev, nullptr, wq_dev, wk_dev, wv_dev,
           (const half_t*)sq_dev, (const half_t*)sk_dev, (const half_t*)sv_dev, block, dim, head_dim, eps, rope_row, (const int*)pos_dev,
           table_positions - 1);
     }
   } else {
     if (norm_w_dev) {
-      decode_qkv_kernel<false, 2, true><<<grid, GEMV_THREADS, lds, st>>>(
-          (half_t*)q_out_dev, k_row, v_row, (const half_t*)x_dev, (const half_t*)norm_w_dev, wq_dev, wk_dev, wv_dev,
-          nullptr, nullptr, nullptr, 0, dim, head_dim, eps, rope_row, (const int*)pos_dev, table_positions - 1);
+      with_x_pieces(dim, [&](auto xn) {
+        decode_qkv_kernel<false, 2, decltype(xn)::value><<<grid, GEMV_THREADS, decltype(xn)::value * 4096, st>>>(
+            (half_t*)q_out_dev, k_row, v_row, (const half_t*)x_dev, (const half_t*)norm_w_dev, wq_dev, wk_dev, wv_dev,
+            nullptr, nullptr, nullptr, 0, dim, head_dim, eps, rope_row, (const int*)pos_dev, table_positions - 1);
+      });
     } else {
-      decode_qkv_kernel<false, 2, false><<<grid, GEMV_THREADS, 0, st>>>(
+      decode_qkv_kernel<false, 2, 0><<<grid, GEMV_THREADS, 0, st>>>(
           (half_t*)q_out_dev, k_row, v_row, (const half_t*)x_dev, nullptr, wq_dev, wk_dev, wv_dev, nullptr, nullptr,
           nullptr, 0, dim, head_dim, eps, rope_row, (const int*)pos_dev, table_positions - 1);
     }
@@ -504,28 +570,31 @@ int lcu_decode_ffn_up(void* out_dev, const void* x_dev, const void* norm_w_dev, 
   LCU_REQUIRE(dim > 0 && dim % 16 == 0 && dim <= 24576 && ffn > 0, "lcu_decode_ffn_up: bad shape dim %d ffn %d", dim,
               ffn);
   const int grid = ffn;
-  const size_t lds = (size_t)dim * 2;
   hipStream_t st = as_stream(stream);
   if (block > 0) {
     int rc = check_quant_args("lcu_decode_ffn_up", s1_dev, dim, block);
     if (rc) return rc;
     LCU_REQUIRE(s3_dev != nullptr, "lcu_decode_ffn_up: quantised weights need scales");
     if (norm_w_dev) {
-      decode_ffn_up_kernel<true, 1, true><<<grid, GEMV_THREADS, lds, st>>>(
-          (half_t*)out_dev, (const half_t*)x_dev, (const half_t*)norm_w_dev, w1_dev, w3_dev, (const half_t*)s1_dev,
-          (const half_t*)s3_dev, block, dim, ffn, eps);
+      with_x_pieces(dim, [&](auto xn) {
+        decode_ffn_up_kernel<true, 1, decltype(xn)::value><<<grid, GEMV_THREADS, decltype(xn)::value * 4096, st>>>(
+            (half_t*)out_dev, (const half_t*)x_dev, (const half_t*)norm_w_dev, w1_dev, w3_dev, (const half_t*)s1_dev,
+            (const half_t*)s3_dev, block, dim, ffn, eps);
+      });
     } else {
-      decode_ffn_up_kernel<true, 1, false><<<grid, GEMV_THREADS, 0, st>>>(
+      decode_ffn_up_kernel<true, 1, 0><<<grid, GEMV_THREADS, 0, st>>>(
           (half_t*)out_dev, (const half_t*)x_dev, nullptr, w1_dev, w3_dev, (const half_t*)s1_dev,
           (const half_t*)s3_dev, block, dim, ffn, eps);
     }
   } else {
     if (norm_w_dev) {
-      decode_ffn_up_kernel<false, 2, true><<<grid, GEMV_THREADS, lds, st>>>(
-          (half_t*)out_dev, (const half_t*)x_dev, (const half_t*)norm_w_dev, w1_dev, w3_dev, nullptr, nullptr, 0, dim,
-          ffn, eps);
+      with_x_pieces(dim, [&](auto xn) {
+        decode_ffn_up_kernel<false, 2, decltype(xn)::value><<<grid, GEMV_THREADS, decltype(xn)::value * 4096, st>>>(
+            (half_t*)out_dev, (const half_t*)x_dev, (const half_t*)norm_w_dev, w1_dev, w3_dev, nullptr, nullptr, 0, dim,
+            ffn, eps);
+      });
     } else {
-      decode_ffn_up_kernel<false, 2, false><<<grid, GEMV_THREADS, 0, st>>>(
+      decode_ffn_up_kernel<false, 2, 0><<<grid, GEMV_THREADS, 0, st>>>(
           (half_t*)out_dev, (const half_t*)x_dev, nullptr, w1_dev, w3_dev, nullptr, nullptr, 0, dim, ffn, eps);
     }
   }
@@ -539,18 +608,21 @@ int lcu_decode_logits(void* logits_dev, const void* x_dev, const void* norm_w_de
   LCU_REQUIRE(dim > 0 && dim % 16 == 0 && dim <= 24576 && n_vocab > 0, "lcu_decode_logits: bad shape dim %d vocab %d",
               dim, n_vocab);
   const int grid = (n_vocab + 1) / 2;
-  const size_t lds = (size_t)dim * 2;
   hipStream_t st = as_stream(stream);
   if (block > 0) {
     int rc = check_quant_args("lcu_decode_logits", sout_dev, dim, block);
     if (rc) return rc;
-    gemv_kernel<true, 2, 1, true><<<grid, GEMV_THREADS, lds, st>>>(
-        (half_t*)logits_dev, (const half_t*)x_dev, (const half_t*)norm_w_dev, wout_dev, (const half_t*)sout_dev, dim,
-        n_vocab, block, 0.0f, eps);
+    with_x_pieces(dim, [&](auto xn) {
+      gemv_kernel<true, 2, 1, decltype(xn)::value><<<grid, GEMV_THREADS, decltype(xn)::value * 4096, st>>>(
+          (half_t*)logits_dev, (const half_t*)x_dev, (const half_t*)norm_w_dev, wout_dev, (const half_t*)sout_dev, dim,
+          n_vocab, block, 0.0f, eps);
+    });
   } else {
-    gemv_kernel<false, 2, 2, true><<<grid, GEMV_THREADS, lds, st>>>(
-        (half_t*)logits_dev, (const half_t*)x_dev, (const half_t*)norm_w_dev, wout_dev, nullptr, dim, n_vocab, 0, 0.0f,
-        eps);
+    with_x_pieces(dim, [&](auto xn) {
+      gemv_kernel<false, 2, 2, decltype(xn)::value><<<grid, GEMV_THREADS, decltype(xn)::value * 4096, st>>>(
+          (half_t*)logits_dev, (const half_t*)x_dev, (const half_t*)norm_w_dev, wout_dev, nullptr, dim, n_vocab, 0,
+          0.0f, eps);
+    });
   }
   LCU_LAUNCH_CHECK();
   return LCU_OK;

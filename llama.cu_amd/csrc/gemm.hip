@@ -335,10 +335,14 @@ __device__ __forceinline__ void wait_vmcnt() {
 // at the same permuted chunk positions a direct fp16 load would have filled -- so a weight is
 // dequantised once per block tile and the fragment path is the fp16 one.  The chunk's scale comes
 // by an ordinary 2-byte load one stage earlier.
-template <int BM, int BN, int WM, int WN, int KS, int NS, bool U8>
+//
+// SPLIT (few rows, so few tiles): the grid holds `splits` workgroups per tile, each taking a
+// contiguous run of the K stages and writing its fp32 sums to part[split][M][N];
+// splitk_reduce_kernel adds them in split order and applies the epilogue.
+template <int BM, int BN, int WM, int WN, int KS, int NS, bool U8, bool SPLIT = false>
 __global__ __launch_bounds__(64 * WM * WN * KS, WM * WN * KS <= 4 ? 2 : 1) void gemm_dl_kernel(
     half_t* __restrict__ out, const half_t* __restrict__ A, const void* __restrict__ W, const half_t* __restrict__ S,
-    int M, int K, int N, int block, float beta, int tiles_m, int tiles_n) {
+    int M, int K, int N, int block, float beta, int tiles_m, int tiles_n, float* __restrict__ part, int splits) {
   constexpr int NG = WM * WN;                // wavefronts of one group
   constexpr int NW = NG * KS;                // wavefronts
   constexpr int BKS = BK * KS;               // K extent of a stage
@@ -373,8 +377,10 @@ __global__ __launch_bounds__(64 * WM * WN * KS, WM * WN * KS <= 4 ? 2 : 1) void 
   const int group = wave / NG, w4 = wave % NG;
   const int wm = (w4 % WM) * (BM / WM), wn = (w4 / WM) * (BN / WN);
   // XCD-aware tile order, as in gemm_kernel
+  const int split = SPLIT ? blockIdx.x / nb : 0;
+  const int bx = SPLIT ? blockIdx.x - split * nb : blockIdx.x;
   const int q = nb / NUM_XCD, r = nb % NUM_XCD;
-  const int xcd = blockIdx.x % NUM_XCD, idx = blockIdx.x / NUM_XCD;
+  const int xcd = bx % NUM_XCD, idx = bx / NUM_XCD;
   const int logical = xcd * q + min(xcd, r) + idx;
   const int tm = logical % tiles_m, tn = logical / tiles_m;
   const int m0 = tm * BM, n0 = tn * BN;
@@ -398,8 +404,13 @@ __global__ __launch_bounds__(64 * WM * WN * KS, WM * WN * KS <= 4 ? 2 : 1) void 
       b_off[j] = ((uint32_t)min(n0 + row, N - 1) * (uint32_t)K + g * 8) * 2u;
     }
   }
-  const char* Ab = (const char*)A;
-  const char* Wb = (const char*)W;
+  // this workgroup's K stages: all of them, or its share [stage0, stage0 + nt) of a split
+  const int nt_all = K / BKS;
+  const int stage0 = SPLIT ? (int)((long)split * nt_all / splits) : 0;
+  const int nt = SPLIT ? (int)((long)(split + 1) * nt_all / splits) - stage0 : nt_all;
+  const int k_base = stage0 * BKS;
+  const char* Ab = (const char*)A + (size_t)k_base * 2;
+  const char* Wb = (const char*)W + (size_t)k_base * (U8 ? 1 : 2);
   // uint8: the chunks this thread dequantises (tile row, chunk in the row), their scale index at
   // stage 0, and where the two fp16 chunks of a dequantised chunk go in the W tile
   int d_scale[DC];
@@ -430,7 +441,6 @@ __global__ __launch_bounds__(64 * WM * WN * KS, WM * WN * KS <= 4 ? 2 : 1) void 
     const uint32_t m0 = __builtin_amdgcn_readfirstlane(lds0 + lds_off);
     asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %0, off" ::"v"(g), "s"(m0) : "memory");
   };
-  const int nt = K / BKS;
   // request `idx` (0 .. P-1) of this wavefront for batch `stage` into ring slot `slot`: the lhs tile
   // of that stage, and the W tile of that stage (fp16) or the codes and scales of the stage after it
   // (uint8; past the end the last stage is fetched again and never used)
@@ -445,7 +455,7 @@ __global__ __launch_bounds__(64 * WM * WN * KS, WM * WN * KS <= 4 ? 2 : 1) void 
       } else {
         const int i = idx - PA - PB;  // the dword that holds this thread's fp16 scale of chunk i
         const int kc = (tid + i * THREADS) % CPR;
-        const int at = d_scale[i] + (st1 * BKS + kc * 16) / block;
+        const int at = d_scale[i] + (k_base + st1 * BKS + kc * 16) / block;
         request4(S + (at & ~1), S_BASE + cslot * S_BYTES + (i * NW + wave) * 256);
       }
     } else {
@@ -483,7 +493,7 @@ __global__ __launch_bounds__(64 * WM * WN * KS, WM * WN * KS <= 4 ? 2 : 1) void 
       const uint4_t q = *reinterpret_cast<const uint4_t*>(gemm_lds + C_BASE + cslot * C_BYTES + d_src[i]);
       const uint32_t pair = *reinterpret_cast<const uint32_t*>(gemm_lds + S_BASE + cslot * S_BYTES + i * THREADS * 4 + tid * 4);
       const int kc = (tid + i * THREADS) % CPR;
-      const int at = d_scale[i] + (stage * BKS + kc * 16) / block;  // the request fetched the dword at (at & ~1)
+      const int at = d_scale[i] + (k_base + stage * BKS + kc * 16) / block;  // the request fetched the dword at (at & ~1)
       const half_t sc = __builtin_bit_cast(half_t, (uint16_t)((at & 1) ? pair >> 16 : pair & 0xffffu));
       const half_t s2 = sc * (half_t)2.0f;
       const half2_t s2v = {s2, s2};
@@ -661,16 +671,59 @@ __global__ __launch_bounds__(64 * WM * WN * KS, WM * WN * KS <= 4 ? 2 : 1) void 
         for (int v = 0; v < 16; ++v) {
           const int gm = m0 + wm + i * 32 + (v >> 2) * 8 + (lane >> 5) * 4 + (v & 3);
           if (gm < M && gn < N) {
-            half_t* p = out + (size_t)gm * N + gn;
-            float val = acc[i][j][v];
-            if (beta != 0.0f) {
-              val = fmaf(beta, (float)*p, val);
+            if constexpr (SPLIT) {
+              part[((size_t)split * M + gm) * N + gn] = acc[i][j][v];
+            } else {
+              half_t* p = out + (size_t)gm * N + gn;
+              float val = acc[i][j][v];
+              if (beta != 0.0f) {
+                val = fmaf(beta, (float)*p, val);
+              }
+              *p = round_f16(val);
             }
-            *p = round_f16(val);
           }
         }
       }
     }
+  }
+}
+
+// out[m][n] = fp16(sum over splits, in split order, of part[s][m][n] + beta * out[m][n])
+__global__ __launch_bounds__(256) void splitk_reduce_kernel(half_t* __restrict__ out, const float* __restrict__ part,
+                                                            size_t mn, int splits, float beta) {
+  const size_t i = ((size_t)blockIdx.x * 256 + threadIdx.x) * 4;
+  if (i >= mn) {
+    return;
+  }
+  if (i + 4 <= mn && mn % 4 == 0) {
+    float4 sum = *reinterpret_cast<const float4*>(part + i);
+    for (int s = 1; s < splits; ++s) {
+      const float4 v = *reinterpret_cast<const float4*>(part + (size_t)s * mn + i);
+      sum.x += v.x;
+      sum.y += v.y;
+      sum.z += v.z;
+      sum.w += v.w;
+    }
+    const float v4[4] = {sum.x, sum.y, sum.z, sum.w};
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      float val = v4[e];
+      if (beta != 0.0f) {
+        val = fmaf(beta, (float)out[i + e], val);
+      }
+      out[i + e] = round_f16(val);
+    }
+    return;
+  }
+  for (size_t j = i; j < min(i + 4, mn); ++j) {
+    float val = part[j];
+    for (int s = 1; s < splits; ++s) {
+      val += part[(size_t)s * mn + j];
+    }
+    if (beta != 0.0f) {
+      val = fmaf(beta, (float)out[j], val);
+    }
+    out[j] = round_f16(val);
   }
 }
 
@@ -694,8 +747,61 @@ int launch_dl(half_t* out, const half_t* A, const void* W, const half_t* S, int 
       raised[dev & 15] = true;
     }
   }
-  kernel<<<tiles_m * tiles_n, 64 * WM * WN * KS, lds, st>>>(out, A, W, S, M, K, N, block, beta, tiles_m, tiles_n);
+  kernel<<<tiles_m * tiles_n, 64 * WM * WN * KS, lds, st>>>(out, A, W, S, M, K, N, block, beta, tiles_m, tiles_n,
+                                                            nullptr, 1);
   LCU_LAUNCH_CHECK();
+  return LCU_OK;
+}
+
+// Few rows (2 .. 64: short prompts, where the reference takes its 16-row tile, llama_cu.cu:1481-1484):
+// BM x 128 tiles with four wavefronts, the K stages split over enough workgroups to give every
+// compute unit one, fp32 partial sums in the per-device workspace, then splitk_reduce_kernel.
+// Returns LCU_OK with *done = false when the shape does not suit it.
+template <int BM, bool U8>
+int launch_skinny(half_t* out, const half_t* A, const void* W, const half_t* S, int M, int K, int N, int block,
+                  float beta, hipStream_t st, bool* done) {
+  // a ring of six stages and 128-wide stages with eight wavefronts measured no faster
+  constexpr int BN = 128, WM = 1, WN = 4, KS = 1, NS = 3;
+  constexpr int ROWB = BK * KS * 2;
+  constexpr int DCH = U8 ? BN * (BK * KS / 16) / (256 * KS) : 0;
+  constexpr size_t lds = (size_t)NS * BM * ROWB + (size_t)(U8 ? 2 : NS) * BN * ROWB +
+                         (U8 ? (size_t)NS * (BN * BK * KS + 256 * KS * 4 * DCH) : 0);
+  static_assert(lds <= 160 * 1024, "LDS");
+  *done = false;
+  device_state* ds = current_device_state();
+  if (ds == nullptr || ds->workspace == nullptr) {
+    return LCU_OK;
+  }
+  const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
+  const int nt_all = K / (BK * KS);
+  // one workgroup per compute unit and at least four stages each: more, shorter splits only add
+  // partial sums (512 workgroups: 16 against 13 us at N = K = 4096)
+  int splits = (ds->compute_units + tiles_m * tiles_n - 1) / (tiles_m * tiles_n);
+  splits = max(1, min(splits, nt_all / 4));
+  const size_t mn = (size_t)M * N;
+  while (splits > 1 && (size_t)splits * mn * sizeof(float) > ds->workspace_bytes) {
+    --splits;
+  }
+  if ((size_t)splits * mn * sizeof(float) > ds->workspace_bytes || (long)tiles_m * tiles_n * splits < ds->compute_units / 2) {
+    return LCU_OK;
+  }
+  auto kernel = gemm_dl_kernel<BM, BN, WM, WN, KS, NS, U8, true>;
+  if constexpr (lds > 64 * 1024) {
+    static bool raised[16] = {};  // per device, once
+    int dev = 0;
+    LCU_HIP(hipGetDevice(&dev));
+    if (!raised[dev & 15]) {
+      LCU_HIP(hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+      raised[dev & 15] = true;
+    }
+  }
+  float* part = (float*)ds->workspace;
+  kernel<<<tiles_m * tiles_n * splits, 256 * KS, lds, st>>>(out, A, W, S, M, K, N, block, beta, tiles_m, tiles_n, part,
+                                                       splits);
+  LCU_LAUNCH_CHECK();
+  splitk_reduce_kernel<<<(unsigned)((mn + 1023) / 1024), 256, 0, st>>>(out, part, mn, splits, beta);
+  LCU_LAUNCH_CHECK();
+  *done = true;
   return LCU_OK;
 }
 
@@ -748,6 +854,19 @@ int dispatch_gemm(half_t* out, const half_t* A, const void* W, const half_t* S, 
   // against 135 us with the register-staged kernel).
   const long tiles128 = (long)((M + 127) / 128) * ((N + 127) / 128);
   const long tiles64 = (long)((M + 127) / 128) * ((N + 63) / 64);
+  if (K % 128 == 0 && M <= 64) {  // short prompts: the weight stream is what counts
+    bool done = false;
+    int rc;
+    if constexpr (U8) {  // 64-row tiles with the code ring would leave LDS for one workgroup only
+      rc = launch_skinny<32, true>(out, A, W, S, M, K, N, block, beta, st, &done);
+    } else {
+      rc = M <= 32 ? launch_skinny<32, false>(out, A, W, S, M, K, N, block, beta, st, &done)
+                   : launch_skinny<64, false>(out, A, W, S, M, K, N, block, beta, st, &done);
+    }
+    if (rc != LCU_OK || done) {
+      return rc;
+    }
+  }
   if (K % 128 == 0) {  // whole stages: the direct-to-LDS kernels
     const long tiles256 = (long)((M + 255) / 256) * ((N + 127) / 128);
     if (tiles256 >= 160) return launch_dl<256, 128, 4, 2, 1, 3, U8>(out, A, W, S, M, K, N, block, beta, st);

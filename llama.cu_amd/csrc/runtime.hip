@@ -49,9 +49,10 @@ int lcu_init(int device) {
                      device, prop.gcnArchName);
   }
   st.compute_units = prop.multiProcessorCount;
-  // per-device workspace for operators that reduce in two launches (lcu_error_stats: 256 x 3
-  // partial sums); calls that use it and overlap on one device race
-  st.workspace_bytes = 4u << 20;
+  // per-device workspace for operators that work in two launches (lcu_error_stats: 256 x 3
+  // partial sums; decode attention over long rows: its scores; GEMMs with few rows: the fp32
+  // partial sums of their K splits); calls that use it and overlap on one device race
+  st.workspace_bytes = 32u << 20;
   LCU_HIP(hipMalloc(&st.workspace, st.workspace_bytes));
   LCU_HIP(hipMemset(st.workspace, 0, st.workspace_bytes));
   LCU_HIP(hipDeviceSynchronize());

@@ -150,10 +150,13 @@ def test_gemv_u8_dequant_is_exact(gpu):
 # the shapes cover every tile configuration of the dispatcher: 128x64 with two wavefront groups,
 # 256x128, 128x128 with eight wavefronts (160..255 tiles: N = 5120), 128x64 with two workgroups per
 # compute unit (N = 4160), 128x128 with four wavefronts (M = 1024, N = 4096), ragged K / M / N, and
-# grids with more tiles than the chip holds workgroups at once (the last three)
+# grids with more tiles than the chip holds workgroups at once ((4096, 128, 4096) .. (2100, 128, 8200)); the
+# last five are short prompts (2..64 rows), which split K over several workgroups per tile: 32- and 64-row
+# tiles, uneven splits (11008 / 64 = 172 stages over 16 workgroups), ragged M and N
 @pytest.mark.parametrize("M,K,N", [(512, 4096, 4096), (512, 4096, 11008), (512, 11008, 4096), (128, 256, 128),
                                    (7, 64, 24), (130, 200, 70), (33, 1024, 257), (512, 256, 5120), (512, 384, 4160),
-                                   (1024, 256, 4096), (500, 128, 5100), (4096, 128, 4096), (512, 256, 17920), (2100, 128, 8200)])
+                                   (1024, 256, 4096), (500, 128, 5100), (4096, 128, 4096), (512, 256, 17920), (2100, 128, 8200),
+                                   (2, 4096, 4096), (17, 1024, 5000), (32, 11008, 4096), (33, 1024, 4100), (64, 4096, 11008)])
 def test_gemm_f16(gpu, M, K, N):
     G = gpu
     x = normal((M, K), 0, 300, 1.0)
@@ -185,7 +188,8 @@ def test_gemm_exact_cases(gpu):
 
 @pytest.mark.parametrize("M,K,N", [(512, 4096, 4096), (512, 4096, 11008), (512, 11008, 4096), (16, 256, 128),
                                    (130, 384, 70), (512, 256, 5120), (512, 384, 4160), (1024, 256, 4096),
-                                   (500, 128, 5100), (40, 384, 300), (4096, 128, 4096), (512, 256, 17920)])
+                                   (500, 128, 5100), (40, 384, 300), (4096, 128, 4096), (512, 256, 17920),
+                                   (5, 4096, 4096), (17, 1024, 5000), (32, 11008, 4096), (64, 1024, 4100)])
 def test_gemm_u8(gpu, M, K, N):
     G = gpu
     x = normal((M, K), 0, 400, 1.0)

@@ -73,7 +73,10 @@ int lcu_event_elapsed_ms(float* out_ms, void* start_event, void* stop_event);   
 /* ---- matmul: out[M,N] = lhs[M,K] * rhs[N,K]^T + beta * out ----
  * lcu_gemm_f16_nt replaces matmul_nt(tensor4d_view) and the kernels it selects
  * (llama_cu.cu:1463-1496, 150-220, 225-285): M == 1 runs the streaming GEMV, larger M the MFMA
- * GEMM.  K must be a multiple of 8.  fp32 accumulation, one rounding to fp16 of acc + beta*out. */
+ * GEMM.  K must be a multiple of 8.  fp32 accumulation, one rounding to fp16 of acc + beta*out.
+ * With 2 <= M <= 64 (short prompts) and K a multiple of 128 the K range is split over workgroups
+ * and the fp32 partial sums pass through the per-device workspace (both GEMM entry points): such
+ * calls that overlap on one device race. */
 int lcu_gemm_f16_nt(void* out_dev, const void* lhs_dev, const void* rhs_dev, int M, int K, int N,
                     float beta, void* stream);
 /* lcu_gemm_f16u8_nt replaces matmul_nt(generic_tensor&) for quantised weights and

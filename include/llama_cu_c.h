@@ -59,6 +59,9 @@ int lcu_context_read_hidden(lcu_context*, uint16_t* out, int rows);
 int lcu_context_read_kv(lcu_context*, int layer, uint16_t* k_out, uint16_t* v_out, int T);
 /* the hipStream_t (as void*) the context launches on, for event timing */
 void* lcu_context_stream(lcu_context*);
+/* llama_context::sample_with_seed / greedy: draw the next tokens from the probabilities (the
+ * sampler the reference leaves commented out, llama_cu.cu:1202-1203) or take the maximum again */
+void lcu_context_set_sampling(lcu_context*, int enabled, uint64_t seed);
 
 /* mapped_buffer(path) + llama_vocabulary(buffer) (main.cpp:25,35; llama_cu.cu:1312-1339).  The
  * file is checked first (entry table and piece offsets inside the file, pieces NUL-terminated):

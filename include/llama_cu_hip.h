@@ -120,6 +120,15 @@ int lcu_argmax_f16(void* out_index_dev, const void* values_dev, int n, void* str
 int lcu_softmax_argmax(void* probs_dev, void* out_index_dev, const void* logits_dev, int n, float temp,
                        void* stream);
 
+/* the sampler the reference leaves commented out at llama_cu.cu:1202-1203
+ * (std::discrete_distribution over the probabilities): int32 index i drawn with probability
+ * p[i] / sum(p) from n fp16 values and 64 random bits, in integer arithmetic (weight = p * 2^24,
+ * r = floor(random * total / 2^64), the smallest i whose running weight sum exceeds r; 0 when all
+ * weights are 0).  random_dev, when not NULL, points at the 64 bits on the device and replaces
+ * `random`, so a captured launch can draw a new number on every replay. */
+int lcu_sample_row(void* out_index_dev, const void* probs_dev, int n, uint64_t random, const void* random_dev,
+                   void* stream);
+
 /* ---- attention: matmul_qk + softmax_rows + matmul_qkv, llama_cu.cu:400-531, launch sites
  * 1161-1171, without the [n_heads, n, T] score tensor in memory.  q [n_new, dim]; k (already
  * rotated) and v are the first T rows of a [*, dim] cache; causal: row r sees columns

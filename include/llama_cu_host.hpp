@@ -203,6 +203,12 @@ struct LLAMA_CU_API llama_context {
   virtual size_t context_memory_usage() = 0;
   virtual short next_token(std::vector<short> const& new_tokens) = 0;
   size_t tokens_left() { return context_len_ - start_pos_; }
+  // Not in the reference, which always returns the most probable token (its sampler,
+  // llama_cu.cu:1202-1203, is commented out): from now on next_token draws the token from the
+  // probabilities (index i with probability p[i] / sum p) with the k-th output of the splitmix64
+  // generator started at `seed` for the k-th token drawn; greedy() returns to the maximum.
+  virtual void sample_with_seed(uint64_t seed) = 0;
+  virtual void greedy() = 0;
 
  protected:
   llama_context(llama_model_impl* model, int context_len, float temperature)

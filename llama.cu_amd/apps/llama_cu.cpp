@@ -1,12 +1,14 @@
 // llama_cu: greedy text generation from a model directory.
 //
-//   llama_cu [matmul_type] [model_name] [prompt] [max_tokens = 200] [context_len = 2048]
+//   llama_cu [matmul_type] [model_name] [prompt] [max_tokens = 200] [context_len = 2048] [sample_seed]
 //
 // The command line, the printed lines, the stop at token 2, the half-context re-prefill when the
 // context is full and the times.txt report follow the reference's main.cpp (9-110); the reference's
 // own main.cpp also builds unchanged against include/llama_cu.h.  matmul_type is accepted and
 // ignored.  A model name is looked up as models/<name>; a name containing '/' is the directory.
-// max_tokens and context_len are additions for testing with small contexts.
+// max_tokens and context_len are additions for testing with small contexts; with sample_seed the
+// tokens are drawn from the probabilities (the sampler the reference leaves commented out,
+// llama_cu.cu:1202-1203) instead of taking the most probable one.
 #include <chrono>
 #include <cstdio>
 #include <cstdlib>
@@ -25,6 +27,8 @@ struct options {
   std::string prompt = "Building a website can be done in 10 easy steps:";
   int max_tokens = 200;
   size_t context_len = 2048;
+  bool sample = false;
+  uint64_t sample_seed = 0;
 };
 
 double seconds_since(steady::time_point t0) { return std::chrono::duration<double>(steady::now() - t0).count(); }
@@ -84,6 +88,10 @@ int main(int argc, char const** argv) {
   if (argc > 3) opt.prompt = argv[3];
   if (argc > 4) opt.max_tokens = atoi(argv[4]);
   if (argc > 5) opt.context_len = (size_t)atol(argv[5]);
+  if (argc > 6) {
+    opt.sample = true;
+    opt.sample_seed = strtoull(argv[6], nullptr, 10);
+  }
   if (opt.context_len < 2) {
     fprintf(stderr, "context_len must be at least 2\n");
     return 1;
@@ -125,6 +133,9 @@ int main(int argc, char const** argv) {
   }
   auto context = llama_context::create(model.get(), (int)opt.context_len, 0.8f);
   printf("Context memory: %f MB\n", context->context_memory_usage() / 1024.0 / 1024.0);
+  if (opt.sample) {
+    context->sample_with_seed(opt.sample_seed);
+  }
 
   const std::vector<short> prompt = vocab.tokenize(opt.prompt, true);
   if (prompt.size() > opt.context_len) {

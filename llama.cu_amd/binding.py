@@ -58,6 +58,7 @@ SIGNATURES = {
     "lcu_embed_u8": (i32, [vp, vp, i32, i32, vp, vp, i32, i32, vp]),
     "lcu_argmax_f16": (i32, [vp, vp, i32, vp]),
     "lcu_softmax_argmax": (i32, [vp, vp, vp, i32, f32, vp]),
+    "lcu_sample_row": (i32, [vp, vp, i32, u64, vp, vp]),
     "lcu_attention": (i32, [vp, vp, vp, vp, i32, i32, i32, i32, i32, vp]),
     "lcu_decode_qkv": (i32, [vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, i32, i32, i32, i32, vp, f32, vp, i32, vp]),
     "lcu_attention_decode": (i32, [vp, vp, vp, vp, vp, i32, i32, i32, vp]),
@@ -90,6 +91,7 @@ SIGNATURES = {
     "lcu_context_read_hidden": (i32, [vp, vp, i32]),
     "lcu_context_read_kv": (i32, [vp, i32, vp, vp, i32]),
     "lcu_context_stream": (vp, [vp]),
+    "lcu_context_set_sampling": (None, [vp, i32, u64]),
     "lcu_vocab_load": (vp, [C.c_char_p]),
     "lcu_vocab_destroy": (None, [vp]),
     "lcu_vocab_size": (i32, [vp]),
@@ -248,6 +250,13 @@ class Context:
 
     def clear_tokens(self):
         lib().lcu_context_clear_tokens(self.h)
+
+    def sample_with_seed(self, seed):
+        """next_token draws from the probabilities from now on (llama_context::sample_with_seed)."""
+        lib().lcu_context_set_sampling(self.h, 1, seed)
+
+    def greedy(self):
+        lib().lcu_context_set_sampling(self.h, 0, 0)
 
     def tokens_left(self):
         return lib().lcu_context_tokens_left(self.h)

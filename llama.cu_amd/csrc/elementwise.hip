@@ -97,6 +97,77 @@ __global__ __launch_bounds__(256) void softmax_rows_kernel(half_t* out, const ha
   }
 }
 
+// Draws index i with probability p[i] / sum(p): the std::discrete_distribution the reference leaves
+// commented out (llama_cu.cu:1202-1203), in integers so that the draw is reproducible bit for bit.
+// weight = p * 2^24 (exact for fp16 in [0, 1]; negative and NaN count 0, values above 65504
+// saturate), r = floor(random * total / 2^64), result = the smallest i whose running sum of weights
+// exceeds r; 0 when every weight is 0.  One workgroup: thread t owns the contiguous run
+// [t * seg, (t + 1) * seg), prefix sums of the run totals across the workgroup, and the thread
+// whose run holds r walks it.
+__device__ __forceinline__ uint64_t sample_weight(half_t h) {
+  const float f = (float)h;
+  if (!(f > 0.0f)) {
+    return 0;
+  }
+  return (uint64_t)(fminf(f, 65504.0f) * 16777216.0f);  // exact: 11 significant bits, at most 2^40
+}
+
+__global__ __launch_bounds__(1024) void sample_row_kernel(int* __restrict__ index, const half_t* __restrict__ probs,
+                                                          int n, uint64_t random, const uint64_t* __restrict__ random_dev) {
+  __shared__ uint64_t wave_total[16];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  if (random_dev) {
+    random = *random_dev;
+  }
+  const int seg = (n + 1023) / 1024;
+  const int begin = min(tid * seg, n), end = min(begin + seg, n);
+  uint64_t own = 0;
+  for (int i = begin; i < end; ++i) {
+    own += sample_weight(probs[i]);
+  }
+  // inclusive prefix over the wavefront, then over the 16 wavefront totals
+  uint64_t incl = own;
+#pragma unroll
+  for (int off = 1; off < 64; off <<= 1) {
+    const uint32_t lo = __shfl_up((uint32_t)incl, off, WAVE), hi = __shfl_up((uint32_t)(incl >> 32), off, WAVE);
+    if (lane >= off) {
+      incl += ((uint64_t)hi << 32) | lo;
+    }
+  }
+  if (lane == 63) {
+    wave_total[wave] = incl;
+  }
+  __syncthreads();
+  uint64_t before = 0, total = 0;
+#pragma unroll
+  for (int w = 0; w < 16; ++w) {
+    if (w < wave) {
+      before += wave_total[w];
+    }
+    total += wave_total[w];
+  }
+  if (total == 0) {
+    if (tid == 0) {
+      *index = 0;
+    }
+    return;
+  }
+  const uint64_t r = __umul64hi(random, total);
+  const uint64_t lo_run = before + incl - own;  // weights in front of this thread's run
+  if (r >= lo_run && r < lo_run + own) {        // exactly one thread: the runs tile [0, total)
+    uint64_t run = lo_run;
+    int pick = end - 1;
+    for (int i = begin; i < end; ++i) {
+      run += sample_weight(probs[i]);
+      if (run > r) {
+        pick = i;
+        break;
+      }
+    }
+    *index = pick;
+  }
+}
+
 // softmax_rows with temperature over one long row (the logits, llama_cu.cu:1196-1197) followed by
 // the first-maximum argmax of the rounded probabilities (1205-1209), in one 1024-thread
 // workgroup with 16-byte loads.  The exponential sum is associated differently from the
@@ -478,6 +549,16 @@ int lcu_softmax_rows(void* out_dev, const void* in_dev, int rows, int w, float t
               (double)temp);
   if (rows == 0) return LCU_OK;
   softmax_rows_kernel<<<rows, 256, 0, as_stream(stream)>>>((half_t*)out_dev, (const half_t*)in_dev, w, temp);
+  LCU_LAUNCH_CHECK();
+  return LCU_OK;
+}
+
+int lcu_sample_row(void* out_index_dev, const void* probs_dev, int n, uint64_t random, const void* random_dev,
+                   void* stream) {
+  LCU_REQUIRE(out_index_dev && probs_dev, "lcu_sample_row: null pointer");
+  LCU_REQUIRE(n > 0 && n <= (1 << 24), "lcu_sample_row: bad length %d", n);
+  sample_row_kernel<<<1, 1024, 0, as_stream(stream)>>>((int*)out_index_dev, (const half_t*)probs_dev, n, random,
+                                                      (const uint64_t*)random_dev);
   LCU_LAUNCH_CHECK();
   return LCU_OK;
 }

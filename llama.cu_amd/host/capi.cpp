@@ -210,6 +210,14 @@ int lcu_context_read_kv(lcu_context* c, int layer, uint16_t* k_out, uint16_t* v_
 
 void* lcu_context_stream(lcu_context* c) { return c->impl()->stream(); }
 
+void lcu_context_set_sampling(lcu_context* c, int enabled, uint64_t seed) {
+  if (enabled) {
+    c->impl()->sample_with_seed(seed);
+  } else {
+    c->impl()->greedy();
+  }
+}
+
 lcu_vocab* lcu_vocab_load(const char* vocab_path) {
   if (!vocab_path) return nullptr;
   mapped_buffer file{std::string(vocab_path)};

@@ -354,6 +354,26 @@ void llama_context_impl::enqueue_head(int n) {
                               stream_));
   // the first maximum of the fp16 probabilities is found on the device; 4 bytes go back to the host
   LCU_CHECK(lcu_softmax_argmax(t_probs_.data(), t_argmax_.data(), t_logits_.data(), vocab, temperature_, stream_));
+  if (sampling_) {  // 1202-1203; the random bits of this step are in t_step_
+    LCU_CHECK(lcu_sample_row(t_argmax_.data(), t_probs_.data(), vocab, 0,
+                             (char*)t_step_.data() + offsetof(step_state, random), stream_));
+  }
+}
+
+void llama_context_impl::sample_with_seed(uint64_t seed) {
+  if (!sampling_) {
+    drop_graph();  // the captured step has no sampler launch
+  }
+  sampling_ = true;
+  sample_seed_ = seed;
+  samples_drawn_ = 0;
+}
+
+void llama_context_impl::greedy() {
+  if (sampling_) {
+    drop_graph();
+  }
+  sampling_ = false;
 }
 
 void llama_context_impl::drop_graph() {
@@ -373,10 +393,19 @@ short llama_context_impl::next_token(std::vector<short> const& new_tokens) {
   const int block = p.q_type == quantization_type::uint8 ? p.quantization_block_size : 0;
   char* x = (char*)t_embed_.data();
   const void* ids = t_tokens_.data();
-  if (n == 1) {
-    host_step_.pos = start_pos_;
-    host_step_.token = new_tokens[0];
+  host_step_.pos = start_pos_;
+  host_step_.token = new_tokens[0];
+  if (sampling_) {  // output samples_drawn_ of splitmix64 started at the seed
+    uint64_t z = sample_seed_ + (samples_drawn_ + 1) * 0x9E3779B97F4A7C15ull;
+    z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+    z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+    host_step_.random = z ^ (z >> 31);
+    ++samples_drawn_;
+  }
+  if (n == 1 || sampling_) {
     LCU_CHECK(lcu_h2d(t_step_.data(), &host_step_, sizeof(host_step_), stream_));
+  }
+  if (n == 1) {
     ids = (char*)t_step_.data() + offsetof(step_state, token);
   } else {
     LCU_CHECK(lcu_h2d(t_tokens_.data(), new_tokens.data(), n * sizeof(short), stream_));  // 1086

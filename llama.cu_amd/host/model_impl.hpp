@@ -41,6 +41,8 @@ struct llama_context_impl final : public llama_context {
   void clear_tokens() override;
   size_t context_memory_usage() override;
   short next_token(std::vector<short> const& new_tokens) override;
+  void sample_with_seed(uint64_t seed) override;
+  void greedy() override;
 
   // read-back used by tests and tools
   llama_model_impl* model() const { return model_; }
@@ -65,14 +67,18 @@ struct llama_context_impl final : public llama_context {
   std::vector<kv_cache_layer> kv_;
   gpu_buffer t_embed_, t_norm_, t_xq_, t_out_, t_w1_, t_w3_, t_silu_;
   gpu_buffer t_tokens_, t_logits_, t_probs_, t_argmax_;
-  // decode step state on the device: {int32 position, int16 token}; the decode kernels read the
-  // position from here, so one captured graph replays for every step
+  // step state on the device: {int32 position, int16 token, 64 random bits}; the decode kernels
+  // and the sampler read it from here, so one captured graph replays for every step
   gpu_buffer t_step_;
   struct step_state {
     int32_t pos;
     int16_t token;
     int16_t pad;
+    uint64_t random;  // this step's 64 random bits when sampling
   } host_step_{};
+  bool sampling_{false};
+  uint64_t sample_seed_{0};
+  uint64_t samples_drawn_{0};
   void* decode_graph_{nullptr};
   int decode_calls_{0};
   int decode_bound_{0};  // the position bound the decode graph was captured with

@@ -439,6 +439,38 @@ void orc_error_stats(float* out3, const uint16_t* a, const uint16_t* b, size_t n
   out3[2] = (float)(sum / (double)n);
 }
 
+static uint64_t sample_weight(uint16_t h) {
+  const float f = h2f(h);
+  if (!(f > 0.0f)) {
+    return 0;  // zero, negative, NaN
+  }
+  const float capped = f < 65504.0f ? f : 65504.0f;
+  return (uint64_t)((double)capped * 16777216.0);  // exact: fp16 values are multiples of 2^-24
+}
+
+int orc_sample_row(const uint16_t* probs, int n, uint64_t random) {
+  uint64_t total = 0;
+  for (int i = 0; i < n; ++i) {
+    total += sample_weight(probs[i]);
+  }
+  if (total == 0) {
+    return 0;
+  }
+  const uint64_t r = (uint64_t)(((unsigned __int128)random * total) >> 64);
+  uint64_t run = 0;
+  for (int i = 0; i < n; ++i) {
+    run += sample_weight(probs[i]);
+    if (run > r) {
+      return i;
+    }
+  }
+  return n - 1;  // not reached: run == total > r
+}
+
+uint64_t orc_step_random(uint64_t seed, uint64_t step) {
+  return splitmix64(seed + step * 0x9E3779B97F4A7C15ull);  // output `step` of the splitmix64 sequence from `seed`
+}
+
 int orc_argmax_first(const uint16_t* probs, int n) {
   int best = 0;
   for (int i = 1; i < n; ++i) {

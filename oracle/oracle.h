@@ -15,7 +15,7 @@
  *   orc_rms_norm, orc_rotary, orc_softmax_rows, orc_silu_mul, orc_matmul_qk, orc_matmul_qkv,
  *   orc_embed[_u8], orc_argmax_first : pinned by closed forms and float64 restatements written
  *       independently in numpy (tests/test_oracle_ops.py).
- *   orc_error_stats : pinned by closed forms (tests/test_oracle_ops.py).
+ *   orc_error_stats, orc_sample_row : pinned by closed forms (tests/test_oracle_ops.py).
  *   orc_context_next_token : pinned by an independent numpy float64 forward pass on a tiny model
  *       (tolerance) and by the prefill-then-decode == longer-prefill invariant.
  * The reference holds no golden vectors for any of these (it has no tests), and its CUDA sources
@@ -78,6 +78,18 @@ void orc_embed_u8(uint16_t* out, const int16_t* ids, int n_ids, int dim, const u
                   const uint16_t* scales, int block);
 /* llama_cu.cu:1205-1209: first maximum of fp16 values compared as float */
 int orc_argmax_first(const uint16_t* probs, int n);
+
+/* Sampler the reference leaves commented out (llama_cu.cu:1202-1203: std::discrete_distribution
+ * over the fp16 probabilities): index i is drawn with probability p[i] / sum(p).  Restated in
+ * integers so that it has one answer: weight[i] = p[i] * 2^24 (exact for every fp16 in [0, 1];
+ * negative and NaN count 0, larger values saturate at 2^24 * 65504), total = sum of the weights,
+ * r = floor(random * total / 2^64), result = the smallest i whose running sum of weights exceeds r
+ * (0 when total is 0).  Pinned by closed forms: one-hot rows, the 1:3 threshold at random = 2^62,
+ * zero weights never drawn, monotone in random, frequencies of a known distribution. */
+int orc_sample_row(const uint16_t* probs, int n, uint64_t random);
+/* the 64 random bits of the `step`-th sampled token of a context seeded with `seed`: output
+ * `step` (from 0) of the splitmix64 generator started at `seed` */
+uint64_t orc_step_random(uint64_t seed, uint64_t step);
 
 /* error_stats, transform.cu:99-150: out3 = {mean of d^2, max |d|, mean |d|}, d = a[i] - b[i] in
  * fp32, sums carried in double (the reference adds fp32 partials with atomics in arrival order,

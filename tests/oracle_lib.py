@@ -45,6 +45,10 @@ def lib():
         L.orc_error_stats.restype = None
         L.orc_argmax_first.argtypes = [vp, i]
         L.orc_argmax_first.restype = i
+        L.orc_sample_row.argtypes = [vp, i, u64]
+        L.orc_sample_row.restype = i
+        L.orc_step_random.argtypes = [u64, u64]
+        L.orc_step_random.restype = u64
         L.orc_model_create.argtypes = [i, i, i, i, i, f, i, i, u64, f]
         L.orc_model_create.restype = vp
         L.orc_model_destroy.argtypes = [vp]
@@ -197,6 +201,15 @@ def error_stats(a, b):
     out = np.empty(3, dtype=np.float32)
     lib().orc_error_stats(_p(out), _p(a), _p(b), a.size)
     return out
+
+
+def sample_row(probs, random):
+    probs = _f16(probs)
+    return lib().orc_sample_row(_p(probs), probs.size, random)
+
+
+def step_random(seed, step):
+    return lib().orc_step_random(seed, step)
 
 
 def argmax_first(probs):

@@ -150,11 +150,13 @@ def test_model_load_failures(models, gpu, tmp_path):
         gpu.P.Model(path=str(bad))
 
 
-def expected_generation(G, model_path, prompt, max_tokens, context_len):
+def expected_generation(G, model_path, prompt, max_tokens, context_len, sample_seed=None):
     """The generation loop of main.cpp:69-100 driven from Python through the C handles."""
     vocab = G.P.Vocabulary(VOCAB)
     model = G.P.Model(path=model_path, context_len=context_len)
     ctx = G.P.Context(model, context_len=context_len, temperature=0.8)
+    if sample_seed is not None:
+        ctx.sample_with_seed(sample_seed)
     feed = vocab.tokenize(prompt, bos=True)
     history, text, n_prompt, generated = list(feed), b"", len(feed), 0
     while generated < max_tokens:
@@ -192,6 +194,20 @@ def test_generation_program(models, gpu, name, max_tokens, context_len):
     times = open(str(root / "times.txt")).read().split()
     assert int(times[0]) == n_prompt and len(times) == 1 + generated
     assert all(float(t) > 0 for t in times[1:])
+
+
+def test_generation_program_with_sample_seed(models, gpu):
+    """The optional sample_seed argument: tokens drawn from the probabilities, reproducibly."""
+    root, _, _ = models
+    prompt = "Building a website"
+    text, _, generated = expected_generation(gpu, str(root / "models" / "tiny"), prompt, 20, 64, sample_seed=77)
+    greedy_text, _, _ = expected_generation(gpu, str(root / "models" / "tiny"), prompt, 20, 64)
+    assert text != greedy_text
+    raw = subprocess.run([os.path.join(BIN, "llama_cu"), "4", "tiny", prompt, "20", "64", "77"], cwd=str(root),
+                         capture_output=True, timeout=300).stdout
+    marker = raw.index(b"Context memory:")
+    body = raw[raw.index(b"\n", marker) + 1:]
+    assert body.startswith(text + ("\ntokens: %d time: " % generated).encode()), (body[:200], text[:200])
 
 
 def test_generation_program_failures(models):

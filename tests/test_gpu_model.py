@@ -147,6 +147,46 @@ def test_context_api_behaviour(gpu):
     assert c.memory_usage() > 2 * 2 * 8 * 256 * 2
 
 
+def test_sampling_follows_the_step_random_sequence(gpu):
+    # llama_context::sample_with_seed: token k is the oracle's draw from the probabilities of step k
+    # with output k of splitmix64(seed); covers the eager step, the captured graph and its replays
+    G = gpu
+    gm = G.P.Model(**SMALL, seed=21, weight_std=0.05)
+    seed = 20240607
+
+    def run(ctx, steps):
+        out, feed = [], [5, 9, 100, 2000, 3]
+        for k in range(steps):
+            tok = ctx.next_token(feed)
+            assert tok == O.sample_row(ctx.probs(), O.step_random(seed, k)), k
+            out.append(tok)
+            feed = [tok]
+        return out
+
+    a = G.P.Context(gm, context_len=64, temperature=1.0)
+    a.sample_with_seed(seed)
+    ta = run(a, 12)
+    greedy = G.P.Context(gm, context_len=64, temperature=1.0)
+    tg, feed = [], [5, 9, 100, 2000, 3]
+    for _ in range(12):
+        tg.append(greedy.next_token(feed))
+        feed = [tg[-1]]
+    assert ta != tg  # at temperature 1 a 2048-way distribution does not keep hitting its mode
+    b = G.P.Context(gm, context_len=64, temperature=1.0)
+    b.sample_with_seed(seed)
+    assert run(b, 12) == ta  # reproducible
+    # back to the maximum: the next token is the argmax of its own probabilities again
+    a.greedy()
+    tok = a.next_token([ta[-1]])
+    assert tok == O.argmax_first(a.probs())
+    # and a restart of the sequence with the same seed
+    a.clear_tokens()
+    a.sample_with_seed(seed)
+    assert run(a, 3) == ta[:3]
+    for o in (a, b, greedy, gm):
+        o.close()
+
+
 def test_one_llama7b_layer_prefill_512_then_decode_at_2048(gpu):
     """One LLaMA-7B decoder layer: 512-token prefill, chunked prefill up to 2047 cached tokens,
     then a single-token decode at KV length 2048."""

@@ -387,6 +387,37 @@ def test_attention_decode_twice_reuses_workspace(gpu):
     G.release()
 
 
+@pytest.mark.parametrize("n", [1, 5, 1000, 1024, 32000, 32003])
+def test_sample_row(gpu, n):
+    # integer arithmetic on both sides: the drawn index must agree exactly
+    G = gpu
+    rng = np.random.default_rng(n)
+    rows = [O.softmax_rows(normal((1, n), 0, 1300 + n, 2.0), 0.8)[0],          # a real distribution
+            (rng.random(n) * 0.01).astype(np.float16),                         # does not sum to 1
+            np.where(rng.random(n) < 0.9, 0, rng.random(n)).astype(np.float16)]  # mostly zeros
+    special = (rng.random(n) * 0.5).astype(np.float16)
+    special[::7] = np.float16(-1.0)
+    special[::11] = np.float16(np.nan)
+    special[n // 2] = np.float16(np.inf)
+    rows.append(special)
+    rows.append(np.zeros(n, dtype=np.float16))
+    randoms = [0, 1, 2**63, 2**64 - 1] + [int(v) for v in rng.integers(0, 2**64, 12, dtype=np.uint64)]
+    idx_d = G.empty((1,), np.int32)
+    for p in rows:
+        pd = G.dev_keep(p)
+        for r in randoms:
+            G.B.check(G.L().lcu_sample_row(idx_d.ptr, pd.ptr, n, r, None, None))
+            assert int(G.host(idx_d, (1,), np.int32)[0]) == O.sample_row(p, r), (n, r)
+    # the random bits read from device memory (what a captured launch does)
+    r = randoms[-1]
+    rd = G.dev_keep(np.array([r], dtype=np.uint64))
+    G.B.check(G.L().lcu_sample_row(idx_d.ptr, G.dev_keep(rows[0]).ptr, n, 0, rd.ptr, None))
+    assert int(G.host(idx_d, (1,), np.int32)[0]) == O.sample_row(rows[0], r)
+    assert G.L().lcu_sample_row(idx_d.ptr, None, n, 0, None, None) == -2
+    assert G.L().lcu_sample_row(idx_d.ptr, rd.ptr, 0, 0, None, None) == -2
+    G.release()
+
+
 @pytest.mark.parametrize("n,temp", [(32000, 0.8), (32003, 0.9), (5, 1.0), (1024, 0.5)])
 def test_softmax_argmax_fused(gpu, n, temp):
     G = gpu

@@ -266,3 +266,44 @@ def test_error_stats_closed_forms():
     want = [np.mean(diff.astype(np.float64) ** 2), np.max(np.abs(diff)), np.mean(np.abs(diff.astype(np.float64)))]
     assert np.allclose(O.error_stats(a, e), want, rtol=1e-6)
     assert np.allclose(O.error_stats(e, a), want, rtol=1e-6)
+
+
+def test_sample_row_closed_forms():
+    # one-hot row: that index for every random number
+    p = np.zeros(100, dtype=np.float16)
+    p[37] = 1.0
+    for r in (0, 1, 2**63, 2**64 - 1):
+        assert O.sample_row(p, r) == 37
+    # weights 1 : 3 -> index 0 exactly while random < 2^62 (r = floor(random * total / 2^64) < weight 0)
+    p = np.array([0.25, 0.75], dtype=np.float16)
+    assert O.sample_row(p, 2**62 - 1) == 0
+    assert O.sample_row(p, 2**62) == 1
+    assert O.sample_row(p, 2**64 - 1) == 1
+    # zero, negative and NaN entries are never drawn; the smallest subnormal (2^-24, weight 1) can be
+    p = np.array([0.0, -1.0, np.nan, 2.0**-24, 0.0, 2.0**-24], dtype=np.float16)
+    seen = {O.sample_row(p, r) for r in range(0, 2**64, 2**64 // 64)}
+    assert seen == {3, 5}
+    assert O.sample_row(p, 2**63 - 1) == 3 and O.sample_row(p, 2**63) == 5
+    # nothing to draw from: index 0
+    assert O.sample_row(np.zeros(10, dtype=np.float16), 12345) == 0
+    # monotone in the random number, and every index of a uniform row is reached in order
+    p = np.full(8, 0.125, dtype=np.float16)
+    idx = [O.sample_row(p, r) for r in range(0, 2**64, 2**64 // 1024)]
+    assert idx == sorted(idx) and [idx.count(k) for k in range(8)] == [128] * 8
+
+
+def test_sample_row_frequencies():
+    # frequencies over the step-random sequence follow p / sum(p) (here sum(p) != 1 on purpose)
+    rng = np.random.default_rng(5)
+    p = rng.random(50).astype(np.float16) * np.float16(0.04)
+    w = p.astype(np.float64) / p.astype(np.float64).sum()
+    n = 20000
+    counts = np.bincount([O.sample_row(p, O.step_random(99, k)) for k in range(n)], minlength=50)
+    # five standard deviations of a binomial count, per index
+    assert (np.abs(counts - n * w) <= 5 * np.sqrt(n * w * (1 - w)) + 1).all()
+
+
+def test_step_random_is_splitmix64():
+    # reference values of the splitmix64 generator seeded with 1234567 (Vigna's test vector)
+    expect = [6457827717110365317, 3203168211198807973, 9817491932198370423, 4593380528125082431, 16408922859458223821]
+    assert [O.step_random(1234567, k) for k in range(5)] == expect

@@ -275,6 +275,26 @@ def cpu_baseline_leg(cfg):
                        % (PROMPT + 2, steps, per_layer * 1e3, head * 1e3, cfg["n_layers"]))
 
 
+def batched_leg(P, model, cfg, sizes=(8, 32), prompt=64, steps=32, warmup=4):
+    """llama_batch_context: aggregate decode tok/s of several sequences stepping together (every weight is
+    read once per step for the whole batch); each sequence starts from its own random prompt."""
+    import time
+    out = {}
+    rng = np.random.default_rng(7)
+    for n_seq in sizes:
+        bc = P.BatchContext(model, n_seq, context_len=512, temperature=0.8)
+        last = [bc.next_token(b, rng.integers(0, cfg["n_vocab"], prompt).astype(np.int16)) for b in range(n_seq)]
+        for _ in range(warmup):
+            last = bc.next_tokens(last)
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            last = bc.next_tokens(last)   # blocks on the tokens coming back, as a serving loop would
+        dt = time.perf_counter() - t0
+        out["sequences_%d" % n_seq] = {"ms_per_step": round(dt / steps * 1e3, 3), "tok_s": round(n_seq * steps / dt, 1)}
+        bc.close()
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -303,6 +323,8 @@ def main():
                  decode_hbm_gb_s=round(dec["bytes_per_token"] / dec["ms_per_step"] / 1e6, 1),
                  decode_frac_of_hbm_roofline=round(dec["bytes_per_token"] / dec["ms_per_step"] / 1e6 / HBM_PEAK_GBS, 3))
     ctx.close()
+    if not args.no_extra:
+        extra["batched_decode"] = batched_leg(P, model, cfg)
     model.close()
     if args.copy_calibration:
         n = 256 << 20

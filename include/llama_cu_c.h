@@ -18,6 +18,7 @@ extern "C" {
 
 typedef struct lcu_model lcu_model;
 typedef struct lcu_context lcu_context;
+typedef struct lcu_batch lcu_batch;
 typedef struct lcu_vocab lcu_vocab;
 
 /* llama_params (llama_cu.h:280-291) from its fields; q_type 0 = fp16, 1 = uint8 */
@@ -62,6 +63,23 @@ void* lcu_context_stream(lcu_context*);
 /* llama_context::sample_with_seed / greedy: draw the next tokens from the probabilities (the
  * sampler the reference leaves commented out, llama_cu.cu:1202-1203) or take the maximum again */
 void lcu_context_set_sampling(lcu_context*, int enabled, uint64_t seed);
+
+/* llama_batch_context (no counterpart in the reference, which lists batching as a TODO,
+ * README.md:34): n_sequences sequences over one model.  lcu_batch_next_token is
+ * lcu_context_next_token on one sequence (prompts); lcu_batch_next_tokens takes one new token per
+ * sequence and writes every sequence's next token, in one pass over the weights.  -1 on bad
+ * arguments (sequence out of range, token outside the vocabulary, a full context). */
+lcu_batch* lcu_batch_create(lcu_model*, int n_sequences, int context_len, float temperature);
+void lcu_batch_destroy(lcu_batch*);
+int lcu_batch_n_sequences(lcu_batch*);
+size_t lcu_batch_memory_usage(lcu_batch*);
+int lcu_batch_clear_tokens(lcu_batch*, int sequence);
+long lcu_batch_tokens_left(lcu_batch*, int sequence);
+int lcu_batch_next_token(lcu_batch*, int sequence, const int16_t* tokens, int n);
+int lcu_batch_next_tokens(lcu_batch*, const int16_t* tokens, int16_t* out_tokens);
+/* fp16 logits / probabilities [n_sequences][n_vocab] of the last lcu_batch_next_tokens */
+int lcu_batch_read_logits(lcu_batch*, uint16_t* out);
+int lcu_batch_read_probs(lcu_batch*, uint16_t* out);
 
 /* mapped_buffer(path) + llama_vocabulary(buffer) (main.cpp:25,35; llama_cu.cu:1312-1339).  The
  * file is checked first (entry table and piece offsets inside the file, pieces NUL-terminated):

@@ -146,6 +146,25 @@ int lcu_attention(void* out_dev, const void* q_dev, const void* k_dev, const voi
 int lcu_attention_decode(void* out_dev, const void* q_dev, const void* k_dev, const void* v_dev,
                          const void* pos_dev, int max_T, int dim, int n_heads, void* stream);
 
+/* ---- one decode step of several sequences (batching is a TODO of the reference, README.md:34):
+ * the GEMMs take the n_seq rows as M; these three handle what differs per sequence.  The caches
+ * are given as device arrays of n_seq pointers ([positions][dim] fp16 each), positions as n_seq
+ * int32 on the device (row pos[b] is the new one of sequence b). ---- */
+/* rotary of row b of q (in place) and of k_new at position pos[b]; rotated k and v_new row b are
+ * stored in row pos[b] of sequence b's caches (launch sites 1144-1156 with a position per row) */
+int lcu_rope_store_batch(void* q_dev, const void* k_new_dev, const void* v_new_dev, const void* k_cache_ptrs_dev,
+                         const void* v_cache_ptrs_dev, const void* pos_dev, int n_seq, int dim, int n_heads,
+                         const void* table_dev, int table_positions, void* stream);
+/* lcu_attention_decode for every sequence in one launch: row b of q against rows 0..pos[b] of
+ * sequence b's caches -> row b of out; max_T bounds pos[b] + 1 */
+int lcu_attention_decode_batch(void* out_dev, const void* q_dev, const void* k_cache_ptrs_dev,
+                               const void* v_cache_ptrs_dev, const void* pos_dev, int n_seq, int max_T, int dim,
+                               int n_heads, void* stream);
+/* lcu_softmax_argmax on `rows` rows of n logits (n a multiple of 8): probabilities [rows][n],
+ * one int32 index per row */
+int lcu_softmax_argmax_rows(void* probs_dev, void* out_index_dev, const void* logits_dev, int rows, int n, float temp,
+                            void* stream);
+
 /* ---- fused decode steps (n_new == 1), each replacing several launch sites of next_token ---- */
 /* rms_norm(x, attn_norm) -> Wq/Wk/Wv GEMV -> RoPE(q, k at position pos) -> q to q_out, k and v into
  * row pos of the caches: llama_cu.cu:1129-1156.  Weight pointers are fp16 [dim, dim], or uint8 codes

@@ -219,6 +219,24 @@ struct LLAMA_CU_API llama_context {
   float temperature_;
 };
 
+// Not in the reference, where batching is a TODO (README.md:34): n_sequences independent sequences
+// over one model.  Each sequence is a llama_context of its own (next_token(sequence, tokens) is that
+// context's next_token: prompts of any length, one sequence at a time); next_tokens advances every
+// sequence by one token in a single pass over the weights, the sequences' rows forming the M of
+// the matrix products.  Greedy (first maximum) tokens, as llama_context returns them.
+struct LLAMA_CU_API llama_batch_context {
+  static std::unique_ptr<llama_batch_context> create(llama_model* model, int n_sequences, int context_len = 2048,
+                                                     float temperature = 0.9);
+  virtual ~llama_batch_context() {}
+  virtual int n_sequences() = 0;
+  virtual void clear_tokens(int sequence) = 0;
+  virtual size_t tokens_left(int sequence) = 0;
+  virtual size_t context_memory_usage() = 0;
+  virtual short next_token(int sequence, std::vector<short> const& new_tokens) = 0;
+  // tokens[b] is the one new token of sequence b; returns the next token of every sequence
+  virtual std::vector<short> next_tokens(std::vector<short> const& tokens) = 0;
+};
+
 LLAMA_CU_API void initialize();
 
 }  // namespace llama_cu

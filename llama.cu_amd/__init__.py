@@ -10,4 +10,4 @@ The directory name contains a dot, so import it by path:
     spec = importlib.util.spec_from_file_location("llama_cu_amd", ".../llama.cu_amd/__init__.py",
                                                   submodule_search_locations=[".../llama.cu_amd"])
 """
-from .binding import (DeviceBuffer, LcuError, Model, Context, Vocabulary, check, from_device, lib, lib_path, to_device)  # noqa: F401
+from .binding import (BatchContext, DeviceBuffer, LcuError, Model, Context, Vocabulary, check, from_device, lib, lib_path, to_device)  # noqa: F401

@@ -59,6 +59,9 @@ SIGNATURES = {
     "lcu_argmax_f16": (i32, [vp, vp, i32, vp]),
     "lcu_softmax_argmax": (i32, [vp, vp, vp, i32, f32, vp]),
     "lcu_sample_row": (i32, [vp, vp, i32, u64, vp, vp]),
+    "lcu_rope_store_batch": (i32, [vp, vp, vp, vp, vp, vp, i32, i32, i32, vp, i32, vp]),
+    "lcu_attention_decode_batch": (i32, [vp, vp, vp, vp, vp, i32, i32, i32, i32, vp]),
+    "lcu_softmax_argmax_rows": (i32, [vp, vp, vp, i32, i32, f32, vp]),
     "lcu_attention": (i32, [vp, vp, vp, vp, i32, i32, i32, i32, i32, vp]),
     "lcu_decode_qkv": (i32, [vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, i32, i32, i32, i32, vp, f32, vp, i32, vp]),
     "lcu_attention_decode": (i32, [vp, vp, vp, vp, vp, i32, i32, i32, vp]),
@@ -92,6 +95,16 @@ SIGNATURES = {
     "lcu_context_read_kv": (i32, [vp, i32, vp, vp, i32]),
     "lcu_context_stream": (vp, [vp]),
     "lcu_context_set_sampling": (None, [vp, i32, u64]),
+    "lcu_batch_create": (vp, [vp, i32, i32, f32]),
+    "lcu_batch_destroy": (None, [vp]),
+    "lcu_batch_n_sequences": (i32, [vp]),
+    "lcu_batch_memory_usage": (sz, [vp]),
+    "lcu_batch_clear_tokens": (i32, [vp, i32]),
+    "lcu_batch_tokens_left": (C.c_long, [vp, i32]),
+    "lcu_batch_next_token": (i32, [vp, i32, vp, i32]),
+    "lcu_batch_next_tokens": (i32, [vp, vp, vp]),
+    "lcu_batch_read_logits": (i32, [vp, vp]),
+    "lcu_batch_read_probs": (i32, [vp, vp]),
     "lcu_vocab_load": (vp, [C.c_char_p]),
     "lcu_vocab_destroy": (None, [vp]),
     "lcu_vocab_size": (i32, [vp]),
@@ -299,6 +312,53 @@ class Context:
             self.close()
         except Exception:
             pass
+
+
+class BatchContext:
+    """llama_batch_context: several sequences over one model, one pass over the weights per step."""
+
+    def __init__(self, model, n_sequences, context_len=2048, temperature=0.9):
+        self.model = model
+        self.n = n_sequences
+        self.h = lib().lcu_batch_create(model.h, n_sequences, context_len, temperature)
+        if not self.h:
+            raise LcuError("batch context creation failed")
+
+    def next_token(self, sequence, tokens):
+        t = np.ascontiguousarray(tokens, dtype=np.int16)
+        return lib().lcu_batch_next_token(self.h, sequence, t.ctypes.data_as(vp), len(t))
+
+    def next_tokens(self, tokens):
+        t = np.ascontiguousarray(tokens, dtype=np.int16)
+        if len(t) != self.n:
+            raise LcuError("one token per sequence")
+        out = np.empty(self.n, dtype=np.int16)
+        check(lib().lcu_batch_next_tokens(self.h, t.ctypes.data_as(vp), out.ctypes.data_as(vp)), "next_tokens")
+        return [int(v) for v in out]
+
+    def clear_tokens(self, sequence):
+        check(lib().lcu_batch_clear_tokens(self.h, sequence), "clear_tokens")
+
+    def tokens_left(self, sequence):
+        return lib().lcu_batch_tokens_left(self.h, sequence)
+
+    def memory_usage(self):
+        return lib().lcu_batch_memory_usage(self.h)
+
+    def logits(self):
+        out = np.empty((self.n, self.model.n_vocab), dtype=np.float16)
+        check(lib().lcu_batch_read_logits(self.h, out.ctypes.data_as(vp)), "read_logits")
+        return out
+
+    def probs(self):
+        out = np.empty((self.n, self.model.n_vocab), dtype=np.float16)
+        check(lib().lcu_batch_read_probs(self.h, out.ctypes.data_as(vp)), "read_probs")
+        return out
+
+    def close(self):
+        if self.h:
+            lib().lcu_batch_destroy(self.h)
+            self.h = None
 
 
 class Vocabulary:

@@ -8,7 +8,7 @@ ROOT = os.path.dirname(PKG)
 LIB = os.path.join(PKG, "libllama_cu_amd.so")
 
 HIP_SOURCES = ["csrc/runtime.hip", "csrc/elementwise.hip", "csrc/gemv.hip", "csrc/gemm.hip", "csrc/attention.hip"]
-HOST_SOURCES = ["host/buffers.cpp", "host/params.cpp", "host/model.cpp", "host/tokenizer.cpp", "host/capi.cpp"]
+HOST_SOURCES = ["host/buffers.cpp", "host/params.cpp", "host/model.cpp", "host/batch.cpp", "host/tokenizer.cpp", "host/capi.cpp"]
 # command line programs linked against the library (found at run time next to bin/ through $ORIGIN)
 APPS = {"transform": "apps/transform.cpp", "llama_cu": "apps/llama_cu.cpp"}
 BIN = os.path.join(PKG, "bin")

@@ -39,10 +39,22 @@ __global__ __launch_bounds__(DEC_THREADS) void decode_attention_kernel(half_t* _
                                                                        const half_t* __restrict__ q,
                                                                        const half_t* __restrict__ k,
                                                                        const half_t* __restrict__ v, int T_cap, int dim,
-                                                                       const int* __restrict__ pos_dev) {
+                                                                       const int* __restrict__ pos_dev,
+                                                                       const half_t* const* __restrict__ k_ptrs,
+                                                                       const half_t* const* __restrict__ v_ptrs) {
   __shared__ half_t sc[MAX_T_DECODE];  // fp16 scores, then fp16 probabilities
   __shared__ float gsum[DEC_GROUPS][HD + 4];
   __shared__ float red[16];
+  // a batch of sequences: blockIdx.y picks the sequence, i.e. its row of q / out, its caches and
+  // its position
+  if (k_ptrs) {
+    const int b = blockIdx.y;
+    k = k_ptrs[b];
+    v = v_ptrs[b];
+    q += (size_t)b * dim;
+    out += (size_t)b * dim;
+    pos_dev += b;
+  }
   const int h = blockIdx.x;
   const int tid = threadIdx.x;
   const int sub = tid & 15, grp = tid >> 4;
@@ -267,7 +279,7 @@ int launch_decode_attention(half_t* out, const half_t* q, const half_t* k, const
   // launch costs more than the spreading saves), beyond that the two launches do (21 us against
   // 28 us at T = 2048)
   if (T_cap <= SINGLE_LAUNCH_MAX_T) {
-    decode_attention_kernel<<<n_heads, DEC_THREADS, 0, s>>>(out, q, k, v, T_cap, dim, pos_dev);
+    decode_attention_kernel<<<n_heads, DEC_THREADS, 0, s>>>(out, q, k, v, T_cap, dim, pos_dev, nullptr, nullptr);
     LCU_LAUNCH_CHECK();
     return LCU_OK;
   }
@@ -528,6 +540,23 @@ int lcu_attention_decode(void* out_dev, const void* q_dev, const void* k_dev, co
   LCU_REQUIRE(max_T > 0 && max_T <= MAX_T_DECODE, "lcu_attention_decode: max_T %d outside 1..%d", max_T, MAX_T_DECODE);
   return launch_decode_attention((half_t*)out_dev, (const half_t*)q_dev, (const half_t*)k_dev, (const half_t*)v_dev,
                                  (const int*)pos_dev, max_T, dim, n_heads, as_stream(stream));
+}
+
+int lcu_attention_decode_batch(void* out_dev, const void* q_dev, const void* k_cache_ptrs_dev,
+                               const void* v_cache_ptrs_dev, const void* pos_dev, int n_seq, int max_T, int dim,
+                               int n_heads, void* stream) {
+  LCU_REQUIRE(out_dev && q_dev && k_cache_ptrs_dev && v_cache_ptrs_dev && pos_dev, "lcu_attention_decode_batch: null pointer");
+  LCU_REQUIRE(n_heads > 0 && n_heads <= MAX_HEADS && dim == n_heads * HD,
+              "lcu_attention_decode_batch: dim %d / heads %d unsupported (head_dim must be 128, at most %d heads)", dim,
+              n_heads, MAX_HEADS);
+  LCU_REQUIRE(max_T > 0 && max_T <= MAX_T_DECODE && n_seq >= 0 && n_seq <= 65535,
+              "lcu_attention_decode_batch: max_T %d outside 1..%d or bad n_seq %d", max_T, MAX_T_DECODE, n_seq);
+  if (n_seq == 0) return LCU_OK;
+  decode_attention_kernel<<<dim3(n_heads, n_seq), DEC_THREADS, 0, as_stream(stream)>>>(
+      (half_t*)out_dev, (const half_t*)q_dev, nullptr, nullptr, max_T, dim, (const int*)pos_dev,
+      (const half_t* const*)k_cache_ptrs_dev, (const half_t* const*)v_cache_ptrs_dev);
+  LCU_LAUNCH_CHECK();
+  return LCU_OK;
 }
 
 }  // extern "C"

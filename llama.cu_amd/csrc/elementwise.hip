@@ -97,6 +97,32 @@ __global__ __launch_bounds__(256) void softmax_rows_kernel(half_t* out, const ha
   }
 }
 
+// One decode step of several sequences at once: row b of q is rotated in place, row b of k_new is
+// rotated and row b of v_new copied into row pos[b] of sequence b's caches (rotary as rope_kernel,
+// llama_cu.cu:368-389 and 1144-1156, with a position per row).  pos is clamped into the table.
+__global__ void rope_store_batch_kernel(half_t* q, const half_t* __restrict__ k_new, const half_t* __restrict__ v_new,
+                                        half_t* const* __restrict__ k_ptrs, half_t* const* __restrict__ v_ptrs,
+                                        const int* __restrict__ pos_dev, int dim, int head_dim,
+                                        const float2* __restrict__ table, int max_pos) {
+  const int pair = blockIdx.x * blockDim.x + threadIdx.x;
+  const int b = blockIdx.y;
+  if (pair * 2 >= dim) return;
+  const int c = pair * 2;
+  const int pos = min(max(pos_dev[b], 0), max_pos);
+  const float2 cs = table[(size_t)pos * (head_dim / 2) + (c % head_dim) / 2];
+  const size_t src = (size_t)b * dim + c, dst = (size_t)pos * dim + c;
+  const half2_t qv = *reinterpret_cast<const half2_t*>(q + src);
+  const half2_t kv = *reinterpret_cast<const half2_t*>(k_new + src);
+  half2_t w;
+  w.x = round_f16(fmaf((float)qv.x, cs.x, -((float)qv.y * cs.y)));
+  w.y = round_f16(fmaf((float)qv.x, cs.y, (float)qv.y * cs.x));
+  *reinterpret_cast<half2_t*>(q + src) = w;
+  w.x = round_f16(fmaf((float)kv.x, cs.x, -((float)kv.y * cs.y)));
+  w.y = round_f16(fmaf((float)kv.x, cs.y, (float)kv.y * cs.x));
+  *reinterpret_cast<half2_t*>(k_ptrs[b] + dst) = w;
+  *reinterpret_cast<half2_t*>(v_ptrs[b] + dst) = *reinterpret_cast<const half2_t*>(v_new + src);
+}
+
 // Draws index i with probability p[i] / sum(p): the std::discrete_distribution the reference leaves
 // commented out (llama_cu.cu:1202-1203), in integers so that the draw is reproducible bit for bit.
 // weight = p * 2^24 (exact for fp16 in [0, 1]; negative and NaN count 0, values above 65504
@@ -177,6 +203,10 @@ __global__ __launch_bounds__(1024) void softmax_argmax_kernel(half_t* __restrict
                                                               const half_t* __restrict__ logits, int n, float temp) {
   __shared__ float sred[16];
   __shared__ int sidx[16];
+  // one row per workgroup (several rows: one sequence of a batch each)
+  probs += (size_t)blockIdx.x * n;
+  logits += (size_t)blockIdx.x * n;
+  index += blockIdx.x;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int n8 = n / 8;
   float m = -INFINITY;
@@ -570,6 +600,36 @@ int lcu_softmax_argmax(void* probs_dev, void* out_index_dev, const void* logits_
   LCU_REQUIRE(probs_dev != logits_dev, "lcu_softmax_argmax: probabilities may not overwrite the logits");
   softmax_argmax_kernel<<<1, 1024, 0, as_stream(stream)>>>((half_t*)probs_dev, (int*)out_index_dev,
                                                           (const half_t*)logits_dev, n, temp);
+  LCU_LAUNCH_CHECK();
+  return LCU_OK;
+}
+
+int lcu_softmax_argmax_rows(void* probs_dev, void* out_index_dev, const void* logits_dev, int rows, int n, float temp,
+                            void* stream) {
+  LCU_REQUIRE(probs_dev && out_index_dev && logits_dev, "lcu_softmax_argmax_rows: null pointer");
+  LCU_REQUIRE(rows >= 0 && n > 0 && n % 8 == 0 && temp > 0.0f, "lcu_softmax_argmax_rows: bad arguments rows %d n %d temp %f",
+              rows, n, (double)temp);
+  LCU_REQUIRE(probs_dev != logits_dev, "lcu_softmax_argmax_rows: probabilities may not overwrite the logits");
+  if (rows == 0) return LCU_OK;
+  softmax_argmax_kernel<<<rows, 1024, 0, as_stream(stream)>>>((half_t*)probs_dev, (int*)out_index_dev,
+                                                             (const half_t*)logits_dev, n, temp);
+  LCU_LAUNCH_CHECK();
+  return LCU_OK;
+}
+
+int lcu_rope_store_batch(void* q_dev, const void* k_new_dev, const void* v_new_dev, const void* k_cache_ptrs_dev,
+                         const void* v_cache_ptrs_dev, const void* pos_dev, int n_seq, int dim, int n_heads,
+                         const void* table_dev, int table_positions, void* stream) {
+  LCU_REQUIRE(q_dev && k_new_dev && v_new_dev && k_cache_ptrs_dev && v_cache_ptrs_dev && pos_dev && table_dev,
+              "lcu_rope_store_batch: null pointer");
+  LCU_REQUIRE(n_seq >= 0 && dim > 0 && n_heads > 0 && dim % n_heads == 0 && (dim / n_heads) % 2 == 0 && table_positions > 0,
+              "lcu_rope_store_batch: bad shape n_seq %d dim %d heads %d", n_seq, dim, n_heads);
+  if (n_seq == 0) return LCU_OK;
+  dim3 grid((dim / 2 + 255) / 256, n_seq);
+  rope_store_batch_kernel<<<grid, 256, 0, as_stream(stream)>>>(
+      (half_t*)q_dev, (const half_t*)k_new_dev, (const half_t*)v_new_dev, (half_t* const*)k_cache_ptrs_dev,
+      (half_t* const*)v_cache_ptrs_dev, (const int*)pos_dev, dim, dim / n_heads, (const float2*)table_dev,
+      table_positions - 1);
   LCU_LAUNCH_CHECK();
   return LCU_OK;
 }

@@ -19,6 +19,15 @@ struct lcu_context {
   llama_context_impl* impl() const { return static_cast<llama_context_impl*>(context.get()); }
 };
 
+struct lcu_batch {
+  std::unique_ptr<llama_batch_context> context;
+  int n_vocab;
+};
+
+namespace llama_cu {
+int batch_context_read(llama_batch_context* ctx, bool probs, uint16_t* out);  // host/batch.cpp
+}
+
 struct lcu_vocab {
   mapped_buffer file;
   std::unique_ptr<llama_vocabulary> vocab;
@@ -209,6 +218,57 @@ int lcu_context_read_kv(lcu_context* c, int layer, uint16_t* k_out, uint16_t* v_
 }
 
 void* lcu_context_stream(lcu_context* c) { return c->impl()->stream(); }
+
+lcu_batch* lcu_batch_create(lcu_model* m, int n_sequences, int context_len, float temperature) {
+  if (!m || n_sequences <= 0 || context_len <= 0 || !(temperature > 0.0f)) {
+    return nullptr;
+  }
+  auto ctx = llama_batch_context::create(m->model.get(), n_sequences, context_len, temperature);
+  if (!ctx) {
+    return nullptr;
+  }
+  return new lcu_batch{std::move(ctx), (int)m->impl()->params.n_vocab};
+}
+
+void lcu_batch_destroy(lcu_batch* b) { delete b; }
+int lcu_batch_n_sequences(lcu_batch* b) { return b->context->n_sequences(); }
+size_t lcu_batch_memory_usage(lcu_batch* b) { return b->context->context_memory_usage(); }
+
+static bool sequence_ok(lcu_batch* b, int sequence) { return b && sequence >= 0 && sequence < b->context->n_sequences(); }
+
+int lcu_batch_clear_tokens(lcu_batch* b, int sequence) {
+  if (!sequence_ok(b, sequence)) return -1;
+  b->context->clear_tokens(sequence);
+  return 0;
+}
+
+long lcu_batch_tokens_left(lcu_batch* b, int sequence) {
+  return sequence_ok(b, sequence) ? (long)b->context->tokens_left(sequence) : -1;
+}
+
+int lcu_batch_next_token(lcu_batch* b, int sequence, const int16_t* tokens, int n) {
+  if (!sequence_ok(b, sequence) || !tokens || n <= 0 || (size_t)n > b->context->tokens_left(sequence)) {
+    return -1;
+  }
+  for (int i = 0; i < n; ++i) {
+    if (tokens[i] < 0 || tokens[i] >= b->n_vocab) return -1;
+  }
+  return b->context->next_token(sequence, std::vector<short>(tokens, tokens + n));
+}
+
+int lcu_batch_next_tokens(lcu_batch* b, const int16_t* tokens, int16_t* out_tokens) {
+  if (!b || !tokens || !out_tokens) return -1;
+  const int n = b->context->n_sequences();
+  for (int i = 0; i < n; ++i) {
+    if (tokens[i] < 0 || tokens[i] >= b->n_vocab || b->context->tokens_left(i) < 1) return -1;
+  }
+  const std::vector<short> out = b->context->next_tokens(std::vector<short>(tokens, tokens + n));
+  for (int i = 0; i < n; ++i) out_tokens[i] = out[i];
+  return 0;
+}
+
+int lcu_batch_read_logits(lcu_batch* b, uint16_t* out) { return batch_context_read(b->context.get(), false, out); }
+int lcu_batch_read_probs(lcu_batch* b, uint16_t* out) { return batch_context_read(b->context.get(), true, out); }
 
 void lcu_context_set_sampling(lcu_context* c, int enabled, uint64_t seed) {
   if (enabled) {

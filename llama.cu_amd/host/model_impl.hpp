@@ -58,6 +58,13 @@ struct llama_context_impl final : public llama_context {
     gpu_buffer v;
   };
   std::vector<kv_cache_layer>& kv() { return kv_; }
+  void* rope_table() const { return rope_table_; }
+  float temperature() const { return temperature_; }
+  // a step taken for this sequence by llama_batch_context: one more cached row
+  void advance_one() {
+    start_pos_ += 1;
+    last_n_ = 1;
+  }
 
  private:
   void matmul(void* out, const void* lhs, weight_tensor const& w, int M, float beta);

@@ -132,6 +132,60 @@ def test_decode_across_the_attention_form_boundary(gpu):
         o.close()
 
 
+@pytest.mark.parametrize("q_type", [0, 1])
+def test_batched_decode_vs_oracle(gpu, q_type):
+    """llama_batch_context: three sequences with prompts of different lengths step together; every
+    sequence's logits and probabilities follow the oracle's own context for that sequence (teacher
+    forced), through the eager step, the captured graph and its replays, a cleared sequence and a
+    sequence that is advanced alone in between."""
+    G = gpu
+    om = O.Model(**SMALL, q_type=q_type, seed=13, weight_std=0.05)
+    gm = G.P.Model(**SMALL, q_type=q_type, seed=13, weight_std=0.05)
+    rng = np.random.default_rng(8)
+    prompts = [rng.integers(0, SMALL["n_vocab"], n).astype(np.int16) for n in (19, 3, 40)]
+    ocs = [O.Context(om, context_len=96, temperature=0.8) for _ in prompts]
+    bc = G.P.BatchContext(gm, 3, context_len=96, temperature=0.8)
+    assert bc.tokens_left(1) == 96 and bc.memory_usage() > 3 * 2 * 2 * 96 * 512 * 2
+    last = []
+    for b, pr in enumerate(prompts):
+        otok = ocs[b].next_token(pr)
+        gtok = bc.next_token(b, pr)
+        last.append(otok)
+        assert bc.tokens_left(b) == 96 - len(pr)
+
+    def step(k):
+        want = [oc.next_token(np.array([t], dtype=np.int16), want=True) for oc, t in zip(ocs, last)]
+        got = bc.next_tokens(last)
+        logits, probs = bc.logits(), bc.probs()
+        for b, (otok, _, ologits, oprobs) in enumerate(want):
+            assert G.max_abs_rel(logits[b], ologits) <= TOL, (k, b)
+            assert G.max_abs_rel(probs[b], oprobs) <= 2 * TOL, (k, b)
+            assert got[b] == O.argmax_first(probs[b])
+            lo = np.sort(ologits.astype(np.float32))
+            if lo[-1] - lo[-2] > 0.05:
+                assert got[b] == otok, (k, b)
+            last[b] = otok
+
+    for k in range(6):
+        step(k)
+    # sequence 1 starts over with a new prompt (new caches), sequence 0 takes two tokens alone
+    bc.clear_tokens(1)
+    ocs[1] = O.Context(om, context_len=96, temperature=0.8)
+    pr = rng.integers(0, SMALL["n_vocab"], 7).astype(np.int16)
+    last[1] = ocs[1].next_token(pr)
+    bc.next_token(1, pr)
+    for _ in range(2):
+        t = np.array([last[0]], dtype=np.int16)
+        last[0] = ocs[0].next_token(t)
+        bc.next_token(0, t)
+    for k in range(6, 11):
+        step(k)
+    assert [bc.tokens_left(b) for b in range(3)] == [96 - 19 - 13, 96 - 7 - 5, 96 - 40 - 11]
+    assert bc.next_token(3, [1]) == -1 and bc.next_token(0, [5000]) == -1
+    bc.close()
+    gm.close()
+
+
 def test_context_api_behaviour(gpu):
     G = gpu
     gm = G.P.Model(**TINY, seed=1)

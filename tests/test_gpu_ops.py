@@ -418,6 +418,61 @@ def test_sample_row(gpu, n):
     G.release()
 
 
+def test_batch_step_operators(gpu):
+    """The per-sequence parts of a batched decode step against their single-sequence forms, bit for bit:
+    rotary + cache append with a position per row, attention over each sequence's own caches, softmax +
+    argmax per row."""
+    G = gpu
+    L = G.L()
+    dim, heads, ctx, B = 512, 4, 40, 3
+    pos = np.array([17, 0, 39], dtype=np.int32)
+    table = G.B.vp()
+    G.B.check(L.lcu_rope_table_create(G.B.C.byref(table), ctx, dim // heads, 10000.0))
+    q, k, v = normal((B, dim), 0, 1500, 1.0), normal((B, dim), 0, 1501, 1.0), normal((B, dim), 0, 1502, 1.0)
+    kc = [normal((ctx, dim), 0, 1510 + b, 1.0) for b in range(B)]
+    vc = [normal((ctx, dim), 0, 1520 + b, 1.0) for b in range(B)]
+    kd, vd = [G.dev_keep(a) for a in kc], [G.dev_keep(a) for a in vc]
+    kptr = G.dev_keep(np.array([d.ptr for d in kd], dtype=np.uint64))
+    vptr = G.dev_keep(np.array([d.ptr for d in vd], dtype=np.uint64))
+    qd, kn, vn, pd = G.dev_keep(q), G.dev_keep(k), G.dev_keep(v), G.dev_keep(pos)
+    G.B.check(L.lcu_rope_store_batch(qd.ptr, kn.ptr, vn.ptr, kptr.ptr, vptr.ptr, pd.ptr, B, dim, heads, table, ctx, None))
+    out_d = G.empty((B, dim))
+    G.B.check(L.lcu_attention_decode_batch(out_d.ptr, qd.ptr, kptr.ptr, vptr.ptr, pd.ptr, B, ctx, dim, heads, None))
+    q_rot, out = G.host(qd, (B, dim)), G.host(out_d, (B, dim))
+    for b in range(B):
+        p = int(pos[b])
+        # single-sequence forms: lcu_rope on the row at its position, lcu_attention_decode on the caches
+        row = G.empty((1, dim))
+        G.B.check(L.lcu_rope(row.ptr, G.dev_keep(q[b:b + 1]).ptr, 1, dim, heads, p, table, ctx, None))
+        assert (G.host(row, (1, dim)).view(np.uint16) == q_rot[b].view(np.uint16)).all()
+        G.B.check(L.lcu_rope(row.ptr, G.dev_keep(k[b:b + 1]).ptr, 1, dim, heads, p, table, ctx, None))
+        k_now, v_now = G.host(kd[b], (ctx, dim)), G.host(vd[b], (ctx, dim))
+        assert (k_now[p].view(np.uint16) == G.host(row, (1, dim))[0].view(np.uint16)).all()
+        assert (v_now[p].view(np.uint16) == v[b].view(np.uint16)).all()
+        others = np.arange(ctx) != p
+        assert (k_now[others].view(np.uint16) == kc[b][others].view(np.uint16)).all()
+        one = G.empty((1, dim))
+        G.B.check(L.lcu_attention_decode(one.ptr, G.dev_keep(q_rot[b:b + 1]).ptr, kd[b].ptr, vd[b].ptr,
+                                         G.dev_keep(pos[b:b + 1]).ptr, ctx, dim, heads, None))
+        assert (G.host(one, (1, dim))[0].view(np.uint16) == out[b].view(np.uint16)).all()
+        # and the oracle on the same caches
+        ref = O.attention(q_rot[b:b + 1], k_now[:p + 1], v_now[:p + 1], heads, p)
+        assert G.max_abs_rel(out[b:b + 1], ref) <= TOL
+    n = 1024
+    x = normal((B, n), 0, 1530, 1.5)
+    probs_d, idx_d = G.empty((B, n)), G.empty((B,), np.int32)
+    G.B.check(L.lcu_softmax_argmax_rows(probs_d.ptr, idx_d.ptr, G.dev_keep(x).ptr, B, n, 0.8, None))
+    probs, idx = G.host(probs_d, (B, n)), G.host(idx_d, (B,), np.int32)
+    p1, i1 = G.empty((n,)), G.empty((1,), np.int32)
+    for b in range(B):
+        G.B.check(L.lcu_softmax_argmax(p1.ptr, i1.ptr, G.dev_keep(x[b:b + 1]).ptr, n, 0.8, None))
+        assert (G.host(p1, (n,)).view(np.uint16) == probs[b].view(np.uint16)).all()
+        assert int(G.host(i1, (1,), np.int32)[0]) == int(idx[b]) == O.argmax_first(probs[b])
+    assert L.lcu_softmax_argmax_rows(probs_d.ptr, idx_d.ptr, G.dev_keep(x).ptr, B, 1001, 0.8, None) == -2
+    assert L.lcu_attention_decode_batch(out_d.ptr, qd.ptr, kptr.ptr, vptr.ptr, pd.ptr, B, ctx, dim, 3, None) == -2
+    G.release()
+
+
 @pytest.mark.parametrize("n,temp", [(32000, 0.8), (32003, 0.9), (5, 1.0), (1024, 0.5)])
 def test_softmax_argmax_fused(gpu, n, temp):
     G = gpu

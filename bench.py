@@ -146,7 +146,8 @@ def ffn_up_kernel_leg(P, cfg, model, ctx, launches):
 
 
 def gemv_leg(P, stream):
-    """BASELINE configs 1 and 2 at M = 1: GB/s of the plain GEMV entry point, weight copies rotated."""
+    """The single matrix-vector products of the benchmark configurations (fp16 and uint8 weights, M = 1): GB/s of
+    the plain GEMV entry point, weight copies rotated."""
     B = P.binding
     L = B.lib()
     out = {}
@@ -194,7 +195,7 @@ def gemv_leg(P, stream):
 
 
 def gemm_leg(P, stream):
-    """512-token prefill GEMMs of BASELINE configs 2 and 3: TFLOP/s against dense fp16 MFMA peak."""
+    """512-token prefill GEMMs of the 7B shapes (fp16 and uint8 weights): TFLOP/s against dense fp16 MFMA peak."""
     B = P.binding
     L = B.lib()
     out = {}

@@ -46,3 +46,20 @@ def test_no_fallback_without_the_library(monkeypatch, tmp_path):
     monkeypatch.setattr(P.binding, "_LIB_PATH", str(tmp_path / "libllama_cu_amd.so"))
     with pytest.raises(P.LcuError):
         P.lib()
+
+
+def test_reference_public_surface_compiles_and_links(tmp_path):
+    """A C++17 program that uses every public name of the reference's header with the reference's
+    signatures builds against include/llama_cu.h and links against the library (g++, no HIP headers)."""
+    import shutil
+    import subprocess
+    if shutil.which("g++") is None:
+        pytest.skip("no g++")
+    exe = tmp_path / "public_surface"
+    lib_dir = os.path.dirname(P.lib_path())
+    cmd = ["g++", "-std=c++17", "-Wall", "-Werror", "-I", os.path.join(ROOT, "include"),
+           os.path.join(ROOT, "tests", "cxx", "public_surface.cpp"), "-L", lib_dir, "-lllama_cu_amd",
+           "-Wl,-rpath," + lib_dir, "-Wl,--allow-shlib-undefined", "-o", str(exe)]
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    assert res.returncode == 0, res.stderr
+    assert exe.exists()

@@ -86,6 +86,15 @@ int lcu_gemm_f16_nt(void* out_dev, const void* lhs_dev, const void* rhs_dev, int
 int lcu_gemm_f16u8_nt(void* out_dev, const void* lhs_dev, const void* codes_dev,
                       const void* scales_dev, int M, int K, int N, int block, float beta,
                       void* stream);
+/* Up to three such products with one lhs and weight matrices of one shape in a single launch
+ * (Wq, Wk, Wv at launch sites 1144-1156; W1, W3 at 1180-1181): out_dev, rhs_dev (codes_dev,
+ * scales_dev) are host arrays of n_mats device pointers.  Same results as n_mats separate calls;
+ * with M == 1 it is n_mats separate calls. */
+int lcu_gemm_f16_nt_multi(void* const* out_dev, const void* lhs_dev, const void* const* rhs_dev, int n_mats, int M,
+                          int K, int N, float beta, void* stream);
+int lcu_gemm_f16u8_nt_multi(void* const* out_dev, const void* lhs_dev, const void* const* codes_dev,
+                            const void* const* scales_dev, int n_mats, int M, int K, int N, int block, float beta,
+                            void* stream);
 
 /* ---- int8 absmax quantiser: transform.cu:28-72 and 74-87; block in {32, 64, 128, 256, 512, 1024} */
 int lcu_quantize_absmax_u8(void* codes_dev, void* scales_dev, const void* in_dev, size_t rows,

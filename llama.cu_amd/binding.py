@@ -59,6 +59,8 @@ SIGNATURES = {
     "lcu_argmax_f16": (i32, [vp, vp, i32, vp]),
     "lcu_softmax_argmax": (i32, [vp, vp, vp, i32, f32, vp]),
     "lcu_sample_row": (i32, [vp, vp, i32, u64, vp, vp]),
+    "lcu_gemm_f16_nt_multi": (i32, [vp, vp, vp, i32, i32, i32, i32, f32, vp]),
+    "lcu_gemm_f16u8_nt_multi": (i32, [vp, vp, vp, vp, i32, i32, i32, i32, i32, f32, vp]),
     "lcu_rope_store_batch": (i32, [vp, vp, vp, vp, vp, vp, i32, i32, i32, vp, i32, vp]),
     "lcu_attention_decode_batch": (i32, [vp, vp, vp, vp, vp, i32, i32, i32, i32, vp]),
     "lcu_softmax_argmax_rows": (i32, [vp, vp, vp, i32, i32, f32, vp]),

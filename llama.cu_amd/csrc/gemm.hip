@@ -34,6 +34,16 @@ namespace {
 constexpr int BK = 64;        // K extent one group of four wavefronts multiplies per stage
 constexpr int NUM_XCD = 8;
 
+// Up to three products lhs * W_g^T with weight matrices of one shape in a single launch (Wq, Wk,
+// Wv; W1, W3): the tile index along N runs through matrix 0, then 1, then 2, `tiles_n_per` tiles
+// each.  Matrix 0 travels in the kernel's ordinary arguments, the others here.
+struct more_matrices_t {
+  half_t* out[2];
+  const void* W[2];
+  const half_t* S[2];
+  int tiles_n_per;  // tiles along N of one matrix; 0: a single matrix
+};
+
 __device__ __forceinline__ half2_t dequant2(uint32_t spread, half2_t scale2x) {
   const uint32_t bits = (spread << 2) | 0x58005800u;                                  // 128 + q/2
   const half2_t t = __builtin_bit_cast(half2_t, bits) - (half2_t)((half_t)191.75f);   // (q - 127.5)/2
@@ -341,8 +351,9 @@ __device__ __forceinline__ void wait_vmcnt() {
 // splitk_reduce_kernel adds them in split order and applies the epilogue.
 template <int BM, int BN, int WM, int WN, int KS, int NS, bool U8, bool SPLIT = false>
 __global__ __launch_bounds__(64 * WM * WN * KS, WM * WN * KS <= 4 ? 2 : 1) void gemm_dl_kernel(
-    half_t* __restrict__ out, const half_t* __restrict__ A, const void* __restrict__ W, const half_t* __restrict__ S,
-    int M, int K, int N, int block, float beta, int tiles_m, int tiles_n, float* __restrict__ part, int splits) {
+    half_t* __restrict__ out0, const half_t* __restrict__ A, const void* __restrict__ W0, const half_t* __restrict__ S0,
+    int M, int K, int N, int block, float beta, int tiles_m, int tiles_n, float* __restrict__ part, int splits,
+    more_matrices_t more) {
   constexpr int NG = WM * WN;                // wavefronts of one group
   constexpr int NW = NG * KS;                // wavefronts
   constexpr int BKS = BK * KS;               // K extent of a stage
@@ -382,7 +393,22 @@ __global__ __launch_bounds__(64 * WM * WN * KS, WM * WN * KS <= 4 ? 2 : 1) void 
   const int q = nb / NUM_XCD, r = nb % NUM_XCD;
   const int xcd = bx % NUM_XCD, idx = bx / NUM_XCD;
   const int logical = xcd * q + min(xcd, r) + idx;
-  const int tm = logical % tiles_m, tn = logical / tiles_m;
+  const int tm = logical % tiles_m;
+  int tn = logical / tiles_m;
+  // which weight matrix this tile belongs to: chosen once, from kernel arguments (scalar selects)
+  half_t* out = out0;
+  const void* W = W0;
+  const half_t* S = S0;
+  if (more.tiles_n_per > 0) {
+    const int g = tn / more.tiles_n_per;
+    tn -= g * more.tiles_n_per;
+    out = g == 0 ? out0 : (g == 1 ? more.out[0] : more.out[1]);
+    W = g == 0 ? W0 : (g == 1 ? more.W[0] : more.W[1]);
+    S = g == 0 ? S0 : (g == 1 ? more.S[0] : more.S[1]);
+    if constexpr (SPLIT) {
+      part += (size_t)g * splits * M * N;  // each matrix has its own partial sums
+    }
+  }
   const int m0 = tm * BM, n0 = tn * BN;
 
   // loader: instruction j of this wavefront fills LDS bytes [(wave + j*NW) * 1024, +1024) of the
@@ -688,9 +714,13 @@ __global__ __launch_bounds__(64 * WM * WN * KS, WM * WN * KS <= 4 ? 2 : 1) void 
   }
 }
 
-// out[m][n] = fp16(sum over splits, in split order, of part[s][m][n] + beta * out[m][n])
-__global__ __launch_bounds__(256) void splitk_reduce_kernel(half_t* __restrict__ out, const float* __restrict__ part,
-                                                            size_t mn, int splits, float beta) {
+// out_g[m][n] = fp16(sum over splits, in split order, of part[g][s][m][n] + beta * out_g[m][n]); blockIdx.y = g
+__global__ __launch_bounds__(256) void splitk_reduce_kernel(half_t* out0, half_t* out1, half_t* out2,
+                                                            const float* __restrict__ part, size_t mn, int splits,
+                                                            float beta) {
+  const int g = blockIdx.y;
+  half_t* out = g == 0 ? out0 : (g == 1 ? out1 : out2);
+  part += (size_t)g * splits * mn;
   const size_t i = ((size_t)blockIdx.x * 256 + threadIdx.x) * 4;
   if (i >= mn) {
     return;
@@ -727,16 +757,29 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(half_t* __restrict__
   }
 }
 
+// the arguments of one launch: matrix 0 and, for fused launches, up to two more of the same shape
+struct operands_t {
+  half_t* out;
+  const void* W;
+  const half_t* S;
+  more_matrices_t more;
+  int n_mats;
+};
+
+inline operands_t single_matrix(half_t* out, const void* W, const half_t* S) {
+  return operands_t{out, W, S, more_matrices_t{{nullptr, nullptr}, {nullptr, nullptr}, {nullptr, nullptr}, 0}, 1};
+}
+
 template <int BM, int BN, int WM, int WN, int KS, int NS, bool U8>
-int launch_dl(half_t* out, const half_t* A, const void* W, const half_t* S, int M, int K, int N, int block,
-              float beta, hipStream_t st) {
+int launch_dl(operands_t op, const half_t* A, int M, int K, int N, int block, float beta, hipStream_t st) {
   constexpr int ROWB = BK * KS * 2;
   constexpr int DCH = U8 ? BN * (BK * KS / 16) / (64 * WM * WN * KS) : 0;  // scale dwords per thread and stage
   constexpr size_t lds = (size_t)NS * BM * ROWB + (size_t)(U8 ? 2 : NS) * BN * ROWB +
                          (U8 ? (size_t)NS * (BN * BK * KS + 64 * WM * WN * KS * 4 * DCH) : 0);
   static_assert(lds <= 160 * 1024, "rings do not fit LDS");
   static_assert(KS == 1 || lds >= (size_t)BM * BN * 4 / 2, "LDS must hold one group's accumulators");
-  const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
+  const int tiles_m = (M + BM - 1) / BM, tiles_n_per = (N + BN - 1) / BN, tiles_n = tiles_n_per * op.n_mats;
+  op.more.tiles_n_per = op.n_mats > 1 ? tiles_n_per : 0;
   auto kernel = gemm_dl_kernel<BM, BN, WM, WN, KS, NS, U8>;
   if constexpr (lds > 64 * 1024) {
     static bool raised[16] = {};  // per device, once
@@ -747,8 +790,8 @@ int launch_dl(half_t* out, const half_t* A, const void* W, const half_t* S, int 
       raised[dev & 15] = true;
     }
   }
-  kernel<<<tiles_m * tiles_n, 64 * WM * WN * KS, lds, st>>>(out, A, W, S, M, K, N, block, beta, tiles_m, tiles_n,
-                                                            nullptr, 1);
+  kernel<<<tiles_m * tiles_n, 64 * WM * WN * KS, lds, st>>>(op.out, A, op.W, op.S, M, K, N, block, beta, tiles_m,
+                                                            tiles_n, nullptr, 1, op.more);
   LCU_LAUNCH_CHECK();
   return LCU_OK;
 }
@@ -758,8 +801,8 @@ int launch_dl(half_t* out, const half_t* A, const void* W, const half_t* S, int 
 // compute unit one, fp32 partial sums in the per-device workspace, then splitk_reduce_kernel.
 // Returns LCU_OK with *done = false when the shape does not suit it.
 template <int BM, bool U8>
-int launch_skinny(half_t* out, const half_t* A, const void* W, const half_t* S, int M, int K, int N, int block,
-                  float beta, hipStream_t st, bool* done) {
+int launch_skinny(operands_t op, const half_t* A, int M, int K, int N, int block, float beta, hipStream_t st,
+                  bool* done) {
   // a ring of six stages and 128-wide stages with eight wavefronts measured no faster
   constexpr int BN = 128, WM = 1, WN = 4, KS = 1, NS = 3;
   constexpr int ROWB = BK * KS * 2;
@@ -772,17 +815,19 @@ int launch_skinny(half_t* out, const half_t* A, const void* W, const half_t* S, 
   if (ds == nullptr || ds->workspace == nullptr) {
     return LCU_OK;
   }
-  const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
+  const int tiles_m = (M + BM - 1) / BM, tiles_n_per = (N + BN - 1) / BN, tiles_n = tiles_n_per * op.n_mats;
+  op.more.tiles_n_per = op.n_mats > 1 ? tiles_n_per : 0;
   const int nt_all = K / (BK * KS);
   // one workgroup per compute unit and at least four stages each: more, shorter splits only add
   // partial sums (512 workgroups: 16 against 13 us at N = K = 4096)
   int splits = (ds->compute_units + tiles_m * tiles_n - 1) / (tiles_m * tiles_n);
   splits = max(1, min(splits, nt_all / 4));
   const size_t mn = (size_t)M * N;
-  while (splits > 1 && (size_t)splits * mn * sizeof(float) > ds->workspace_bytes) {
+  while (splits > 1 && (size_t)splits * mn * op.n_mats * sizeof(float) > ds->workspace_bytes) {
     --splits;
   }
-  if ((size_t)splits * mn * sizeof(float) > ds->workspace_bytes || (long)tiles_m * tiles_n * splits < ds->compute_units / 2) {
+  if ((size_t)splits * mn * op.n_mats * sizeof(float) > ds->workspace_bytes ||
+      (long)tiles_m * tiles_n * splits < ds->compute_units / 2) {
     return LCU_OK;
   }
   auto kernel = gemm_dl_kernel<BM, BN, WM, WN, KS, NS, U8, true>;
@@ -796,10 +841,11 @@ int launch_skinny(half_t* out, const half_t* A, const void* W, const half_t* S, 
     }
   }
   float* part = (float*)ds->workspace;
-  kernel<<<tiles_m * tiles_n * splits, 256 * KS, lds, st>>>(out, A, W, S, M, K, N, block, beta, tiles_m, tiles_n, part,
-                                                       splits);
+  kernel<<<tiles_m * tiles_n * splits, 256 * KS, lds, st>>>(op.out, A, op.W, op.S, M, K, N, block, beta, tiles_m, tiles_n,
+                                                            part, splits, op.more);
   LCU_LAUNCH_CHECK();
-  splitk_reduce_kernel<<<(unsigned)((mn + 1023) / 1024), 256, 0, st>>>(out, part, mn, splits, beta);
+  splitk_reduce_kernel<<<dim3((unsigned)((mn + 1023) / 1024), op.n_mats), 256, 0, st>>>(
+      op.out, op.more.out[0], op.more.out[1], part, mn, splits, beta);
   LCU_LAUNCH_CHECK();
   *done = true;
   return LCU_OK;
@@ -841,8 +887,7 @@ int launch_gemm(half_t* out, const half_t* A, const void* W, const half_t* S, in
 }
 
 template <bool U8>
-int dispatch_gemm(half_t* out, const half_t* A, const void* W, const half_t* S, int M, int K, int N, int block,
-                  float beta, hipStream_t st) {
+int dispatch_gemm(operands_t op, const half_t* A, int M, int K, int N, int block, float beta, hipStream_t st) {
   // Tile choice.  Large tiles read fewer operand bytes per multiply-add, and the per-CU load path
   // is what these kernels run against; but a compute unit needs two wavefronts per SIMD to overlap
   // LDS waits with matrix work.  So: 256x128 tiles with eight wavefronts when that still gives 160
@@ -852,36 +897,54 @@ int dispatch_gemm(half_t* out, const half_t* A, const void* W, const half_t* S, 
   // with two groups of four wavefronts splitting the K stage, because then the grid cannot give a
   // compute unit a second workgroup (M = 512, N = 4096: 35 us against 41 us, K = 11008: 100 us
   // against 135 us with the register-staged kernel).
-  const long tiles128 = (long)((M + 127) / 128) * ((N + 127) / 128);
-  const long tiles64 = (long)((M + 127) / 128) * ((N + 63) / 64);
+  // Several matrices of one shape (op.n_mats > 1) count as one product with n_mats * N columns.
+  const long nm = op.n_mats;
+  const long tiles128 = (long)((M + 127) / 128) * ((N + 127) / 128) * nm;
+  const long tiles64 = (long)((M + 127) / 128) * ((N + 63) / 64) * nm;
   if (K % 128 == 0 && M <= 64) {  // short prompts: the weight stream is what counts
     bool done = false;
     int rc;
     if constexpr (U8) {  // 64-row tiles with the code ring would leave LDS for one workgroup only
-      rc = launch_skinny<32, true>(out, A, W, S, M, K, N, block, beta, st, &done);
+      rc = launch_skinny<32, true>(op, A, M, K, N, block, beta, st, &done);
     } else {
-      rc = M <= 32 ? launch_skinny<32, false>(out, A, W, S, M, K, N, block, beta, st, &done)
-                   : launch_skinny<64, false>(out, A, W, S, M, K, N, block, beta, st, &done);
+      rc = M <= 32 ? launch_skinny<32, false>(op, A, M, K, N, block, beta, st, &done)
+                   : launch_skinny<64, false>(op, A, M, K, N, block, beta, st, &done);
     }
     if (rc != LCU_OK || done) {
       return rc;
     }
   }
   if (K % 128 == 0) {  // whole stages: the direct-to-LDS kernels
-    const long tiles256 = (long)((M + 255) / 256) * ((N + 127) / 128);
-    if (tiles256 >= 160) return launch_dl<256, 128, 4, 2, 1, 3, U8>(out, A, W, S, M, K, N, block, beta, st);
+    const long tiles256 = (long)((M + 255) / 256) * ((N + 127) / 128) * nm;
+    if (tiles256 >= 160) return launch_dl<256, 128, 4, 2, 1, 3, U8>(op, A, M, K, N, block, beta, st);
     if constexpr (!U8) {  // uint8 needs a code ring and two W tiles besides: too much LDS for two workgroups
-      if (tiles128 >= 256) return launch_dl<128, 128, 2, 2, 1, 2, false>(out, A, W, S, M, K, N, block, beta, st);
+      if (tiles128 >= 256) return launch_dl<128, 128, 2, 2, 1, 2, false>(op, A, M, K, N, block, beta, st);
     }
     if (tiles128 < 256) {
-      if (tiles128 >= 160) return launch_dl<128, 128, 4, 2, 1, 3, U8>(out, A, W, S, M, K, N, block, beta, st);
-      if (tiles64 > 256) return launch_dl<128, 64, 2, 2, 1, 3, U8>(out, A, W, S, M, K, N, block, beta, st);
-      return launch_dl<128, 64, 2, 2, 2, 3, U8>(out, A, W, S, M, K, N, block, beta, st);
+      if (tiles128 >= 160) return launch_dl<128, 128, 4, 2, 1, 3, U8>(op, A, M, K, N, block, beta, st);
+      if (tiles64 > 256) return launch_dl<128, 64, 2, 2, 1, 3, U8>(op, A, M, K, N, block, beta, st);
+      return launch_dl<128, 64, 2, 2, 2, 3, U8>(op, A, M, K, N, block, beta, st);
     }
   }
-  if (tiles128 >= 256) return launch_gemm<128, 128, U8, 1>(out, A, W, S, M, K, N, block, beta, st);
-  if (tiles64 > 256) return launch_gemm<128, 64, U8, 1>(out, A, W, S, M, K, N, block, beta, st);
-  return launch_gemm<128, 64, U8, 2>(out, A, W, S, M, K, N, block, beta, st);
+  // ragged K: the register-staged kernel, one matrix per launch
+  for (int g = 0; g < op.n_mats; ++g) {
+    half_t* out = g == 0 ? op.out : op.more.out[g - 1];
+    const void* W = g == 0 ? op.W : op.more.W[g - 1];
+    const half_t* S = g == 0 ? op.S : op.more.S[g - 1];
+    const long t128 = tiles128 / nm, t64 = tiles64 / nm;
+    int rc;
+    if (t128 >= 256) {
+      rc = launch_gemm<128, 128, U8, 1>(out, A, W, S, M, K, N, block, beta, st);
+    } else if (t64 > 256) {
+      rc = launch_gemm<128, 64, U8, 1>(out, A, W, S, M, K, N, block, beta, st);
+    } else {
+      rc = launch_gemm<128, 64, U8, 2>(out, A, W, S, M, K, N, block, beta, st);
+    }
+    if (rc != LCU_OK) {
+      return rc;
+    }
+  }
+  return LCU_OK;
 }
 
 }  // namespace
@@ -899,8 +962,35 @@ int lcu_gemm_f16_nt(void* out_dev, const void* lhs_dev, const void* rhs_dev, int
   if (M == 1 && K <= 24576) {
     return gemv_f16((half_t*)out_dev, (const half_t*)lhs_dev, (const half_t*)rhs_dev, K, N, beta, as_stream(stream));
   }
-  return dispatch_gemm<false>((half_t*)out_dev, (const half_t*)lhs_dev, rhs_dev, nullptr, M, K, N, 0, beta,
+  return dispatch_gemm<false>(single_matrix((half_t*)out_dev, rhs_dev, nullptr), (const half_t*)lhs_dev, M, K, N, 0, beta,
                               as_stream(stream));
+}
+
+int lcu_gemm_f16_nt_multi(void* const* out_dev, const void* lhs_dev, const void* const* rhs_dev, int n_mats, int M,
+                          int K, int N, float beta, void* stream) {
+  LCU_REQUIRE(out_dev && lhs_dev && rhs_dev && n_mats >= 1 && n_mats <= 3, "lcu_gemm_f16_nt_multi: bad arguments");
+  for (int g = 0; g < n_mats; ++g) {
+    LCU_REQUIRE(out_dev[g] && rhs_dev[g], "lcu_gemm_f16_nt_multi: null pointer");
+  }
+  if (M == 1 || n_mats == 1) {  // matrix-vector products and single matrices: the ordinary entry point
+    for (int g = 0; g < n_mats; ++g) {
+      const int rc = lcu_gemm_f16_nt(out_dev[g], lhs_dev, rhs_dev[g], M, K, N, beta, stream);
+      if (rc != LCU_OK) return rc;
+    }
+    return LCU_OK;
+  }
+  LCU_REQUIRE(M >= 0 && N > 0 && K > 0 && K % 8 == 0, "lcu_gemm_f16_nt_multi: bad shape M %d K %d N %d (K %% 8 == 0)", M,
+              K, N);
+  if (M == 0) return LCU_OK;
+  LCU_REQUIRE((size_t)M * K * 2 < ((size_t)1 << 32) && (size_t)N * K * 2 < ((size_t)1 << 32),
+              "lcu_gemm_f16_nt_multi: operands of 4 GiB or more are not supported");
+  operands_t op = single_matrix((half_t*)out_dev[0], rhs_dev[0], nullptr);
+  op.n_mats = n_mats;
+  for (int g = 1; g < n_mats; ++g) {
+    op.more.out[g - 1] = (half_t*)out_dev[g];
+    op.more.W[g - 1] = rhs_dev[g];
+  }
+  return dispatch_gemm<false>(op, (const half_t*)lhs_dev, M, K, N, 0, beta, as_stream(stream));
 }
 
 int lcu_gemm_f16u8_nt(void* out_dev, const void* lhs_dev, const void* codes_dev, const void* scales_dev, int M,
@@ -916,8 +1006,38 @@ int lcu_gemm_f16u8_nt(void* out_dev, const void* lhs_dev, const void* codes_dev,
     return gemv_u8((half_t*)out_dev, (const half_t*)lhs_dev, (const uint8_t*)codes_dev, (const half_t*)scales_dev, K,
                    N, block, beta, as_stream(stream));
   }
-  return dispatch_gemm<true>((half_t*)out_dev, (const half_t*)lhs_dev, codes_dev, (const half_t*)scales_dev, M, K, N,
-                             block, beta, as_stream(stream));
+  return dispatch_gemm<true>(single_matrix((half_t*)out_dev, codes_dev, (const half_t*)scales_dev), (const half_t*)lhs_dev,
+                             M, K, N, block, beta, as_stream(stream));
+}
+
+int lcu_gemm_f16u8_nt_multi(void* const* out_dev, const void* lhs_dev, const void* const* codes_dev,
+                            const void* const* scales_dev, int n_mats, int M, int K, int N, int block, float beta,
+                            void* stream) {
+  LCU_REQUIRE(out_dev && lhs_dev && codes_dev && scales_dev && n_mats >= 1 && n_mats <= 3,
+              "lcu_gemm_f16u8_nt_multi: bad arguments");
+  for (int g = 0; g < n_mats; ++g) {
+    LCU_REQUIRE(out_dev[g] && codes_dev[g] && scales_dev[g], "lcu_gemm_f16u8_nt_multi: null pointer");
+  }
+  if (M == 1 || n_mats == 1) {
+    for (int g = 0; g < n_mats; ++g) {
+      const int rc = lcu_gemm_f16u8_nt(out_dev[g], lhs_dev, codes_dev[g], scales_dev[g], M, K, N, block, beta, stream);
+      if (rc != LCU_OK) return rc;
+    }
+    return LCU_OK;
+  }
+  LCU_REQUIRE(M >= 0 && N > 0 && K > 0 && K % 16 == 0 && block >= 16 && block % 16 == 0 && K % block == 0,
+              "lcu_gemm_f16u8_nt_multi: bad shape M %d K %d N %d block %d", M, K, N, block);
+  if (M == 0) return LCU_OK;
+  LCU_REQUIRE((size_t)M * K * 2 < ((size_t)1 << 32) && (size_t)N * K < ((size_t)1 << 32),
+              "lcu_gemm_f16u8_nt_multi: operands of 4 GiB or more are not supported");
+  operands_t op = single_matrix((half_t*)out_dev[0], codes_dev[0], (const half_t*)scales_dev[0]);
+  op.n_mats = n_mats;
+  for (int g = 1; g < n_mats; ++g) {
+    op.more.out[g - 1] = (half_t*)out_dev[g];
+    op.more.W[g - 1] = codes_dev[g];
+    op.more.S[g - 1] = (const half_t*)scales_dev[g];
+  }
+  return dispatch_gemm<true>(op, (const half_t*)lhs_dev, M, K, N, block, beta, as_stream(stream));
 }
 
 }  // extern "C"

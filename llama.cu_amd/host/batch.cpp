@@ -154,6 +154,22 @@ struct llama_batch_context_impl final : public llama_batch_context {
     }
   }
 
+  void matmul_multi(void* const* outs, const void* lhs, weight_tensor const* const* ws, int count, int M) {
+    const void* values[3];
+    const void* scales[3];
+    for (int g = 0; g < count; ++g) {
+      values[g] = ws[g]->data.data();
+      scales[g] = ws[g]->scales.data();
+    }
+    weight_tensor const& w = *ws[0];
+    if (w.quantised) {
+      LCU_CHECK(lcu_gemm_f16u8_nt_multi(outs, lhs, values, scales, count, M, (int)w.cols, (int)w.rows, w.block, 0.0f,
+                                        stream_));
+    } else {
+      LCU_CHECK(lcu_gemm_f16_nt_multi(outs, lhs, values, count, M, (int)w.cols, (int)w.rows, 0.0f, stream_));
+    }
+  }
+
   void enqueue_step(int bound) {
     llama_params const& p = model_->params;
     const int B = (int)seqs_.size(), dim = p.dim, ffn = p.ffn_dim(), heads = p.n_heads, vocab = p.n_vocab;
@@ -172,17 +188,18 @@ struct llama_batch_context_impl final : public llama_batch_context {
       const char* kp = (char*)t_cache_ptrs_.data() + (l * 2 + 0) * B * sizeof(void*);
       const char* vp = (char*)t_cache_ptrs_.data() + (l * 2 + 1) * B * sizeof(void*);
       LCU_CHECK(lcu_rmsnorm(t_norm_.data(), x, L.attn_norm.data(), B, dim, p.norm_eps, stream_));         // 1129
-      matmul(t_q_.data(), t_norm_.data(), L.wq, B, 0.0f);                                                  // 1144
-      matmul(t_k_.data(), t_norm_.data(), L.wk, B, 0.0f);                                                  // 1150
-      matmul(t_v_.data(), t_norm_.data(), L.wv, B, 0.0f);                                                  // 1156
+      void* const qkv_out[3] = {t_q_.data(), t_k_.data(), t_v_.data()};
+      weight_tensor const* const qkv_w[3] = {&L.wq, &L.wk, &L.wv};
+      matmul_multi(qkv_out, t_norm_.data(), qkv_w, 3, B);                                                  // 1144, 1150, 1156
       LCU_CHECK(lcu_rope_store_batch(t_q_.data(), t_k_.data(), t_v_.data(), kp, vp, pos, B, dim, heads,
                                      seqs_[0]->rope_table(), context_len_, stream_));                      // 1146, 1152
       LCU_CHECK(lcu_attention_decode_batch(t_out_.data(), t_q_.data(), kp, vp, pos, B, bound, dim, heads,
                                            stream_));                                                      // 1161-1171
       matmul(x, t_out_.data(), L.wo, B, 1.0f);                                                             // 1174
       LCU_CHECK(lcu_rmsnorm(t_norm_.data(), x, L.ffn_norm.data(), B, dim, p.norm_eps, stream_));          // 1176
-      matmul(t_w1_.data(), t_norm_.data(), L.w1, B, 0.0f);                                                 // 1180
-      matmul(t_w3_.data(), t_norm_.data(), L.w3, B, 0.0f);                                                 // 1181
+      void* const up_out[2] = {t_w1_.data(), t_w3_.data()};
+      weight_tensor const* const up_w[2] = {&L.w1, &L.w3};
+      matmul_multi(up_out, t_norm_.data(), up_w, 2, B);                                                    // 1180, 1181
       LCU_CHECK(lcu_silu_mul(t_silu_.data(), t_w1_.data(), t_w3_.data(), (size_t)B * ffn, stream_));      // 1183
       matmul(x, t_silu_.data(), L.w2, B, 1.0f);                                                            // 1185
     }

@@ -296,6 +296,24 @@ void llama_context_impl::matmul(void* out, const void* lhs, weight_tensor const&
   }
 }
 
+// products of one lhs with several weight matrices of one shape (Wq, Wk, Wv; W1, W3) in one launch
+void llama_context_impl::matmul_multi(void* const* outs, const void* lhs, weight_tensor const* const* ws, int count,
+                                      int M) {
+  const void* values[3];
+  const void* scales[3];
+  for (int g = 0; g < count; ++g) {
+    values[g] = ws[g]->data.data();
+    scales[g] = ws[g]->scales.data();
+  }
+  weight_tensor const& w = *ws[0];
+  if (w.quantised) {
+    LCU_CHECK(lcu_gemm_f16u8_nt_multi(outs, lhs, values, scales, count, M, (int)w.cols, (int)w.rows, w.block, 0.0f,
+                                      stream_));
+  } else {
+    LCU_CHECK(lcu_gemm_f16_nt_multi(outs, lhs, values, count, M, (int)w.cols, (int)w.rows, 0.0f, stream_));
+  }
+}
+
 // The layer loop for n new rows sitting in t_embed_; positions start_pos_ .. start_pos_ + n - 1.
 // n == 1 takes the fused decode kernels, which read the position from t_step_ on the device.
 void llama_context_impl::enqueue_layers(int n) {
@@ -320,11 +338,11 @@ void llama_context_impl::enqueue_layers(int n) {
       char* k_new = kc + (size_t)sp * dim * 2;
       char* v_new = vc + (size_t)sp * dim * 2;
       LCU_CHECK(lcu_rmsnorm(t_norm_.data(), x, L.attn_norm.data(), n, dim, p.norm_eps, stream_));            // 1129
-      matmul(t_xq_.data(), t_norm_.data(), L.wq, n, 0.0f);                                                   // 1144
+      void* const qkv_out[3] = {t_xq_.data(), k_new, v_new};
+      weight_tensor const* const qkv_w[3] = {&L.wq, &L.wk, &L.wv};
+      matmul_multi(qkv_out, t_norm_.data(), qkv_w, 3, n);                                                    // 1144, 1150, 1156
       LCU_CHECK(lcu_rope(t_xq_.data(), t_xq_.data(), n, dim, heads, sp, rope_table_, context_len_, stream_));  // 1146
-      matmul(k_new, t_norm_.data(), L.wk, n, 0.0f);                                                          // 1150
       LCU_CHECK(lcu_rope(k_new, k_new, n, dim, heads, sp, rope_table_, context_len_, stream_));  // 1152, new rows only
-      matmul(v_new, t_norm_.data(), L.wv, n, 0.0f);                                                          // 1156
       LCU_CHECK(lcu_attention(t_out_.data(), t_xq_.data(), kc, vc, n, T, sp, dim, heads, stream_));          // 1161-1171
     }
     matmul(x, t_out_.data(), L.wo, n, 1.0f);                                                                 // 1174
@@ -334,8 +352,9 @@ void llama_context_impl::enqueue_layers(int n) {
       LCU_CHECK(lcu_decode_ffn_up(t_silu_.data(), t_norm_.data(), nullptr, L.w1.data.data(), L.w3.data.data(),
                                   L.w1.scales.data(), L.w3.scales.data(), block, dim, ffn, p.norm_eps, stream_));
     } else {
-      matmul(t_w1_.data(), t_norm_.data(), L.w1, n, 0.0f);                                                   // 1180
-      matmul(t_w3_.data(), t_norm_.data(), L.w3, n, 0.0f);                                                   // 1181
+      void* const up_out[2] = {t_w1_.data(), t_w3_.data()};
+      weight_tensor const* const up_w[2] = {&L.w1, &L.w3};
+      matmul_multi(up_out, t_norm_.data(), up_w, 2, n);                                                      // 1180, 1181
       LCU_CHECK(lcu_silu_mul(t_silu_.data(), t_w1_.data(), t_w3_.data(), (size_t)n * ffn, stream_));         // 1183
     }
     matmul(x, t_silu_.data(), L.w2, n, 1.0f);                                                                // 1185

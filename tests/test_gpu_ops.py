@@ -205,6 +205,45 @@ def test_gemm_u8(gpu, M, K, N):
     G.release()
 
 
+@pytest.mark.parametrize("M,K,N,count", [(512, 512, 4096, 3), (8, 4096, 4096, 3), (40, 1024, 11008, 2), (300, 256, 700, 2),
+                                          (33, 200, 70, 3), (1, 512, 300, 3)])
+def test_gemm_multi_matches_separate_calls(gpu, M, K, N, count):
+    """Several weight matrices of one shape in one launch (Wq, Wk, Wv; W1, W3): what separate calls give
+    (to the matmul tolerance: the fused launch may pick another tile shape, hence another summation order)
+    and what the oracle gives, for fp16 and uint8 weights, in every dispatch branch (large tiles,
+    short-prompt split-K, ragged K, a single row)."""
+    G = gpu
+    L = G.L()
+    VP = G.B.vp
+    x = normal((M, K), 0, 1600, 1.0)
+    xd = G.dev_keep(x)
+    ws = [normal((N, K), 0, 1601 + g, 0.02) for g in range(count)]
+    wd = [G.dev_keep(w) for w in ws]
+    sep = [G.gemm_f16(x, w) for w in ws]
+    outs = [G.empty((M, N)) for _ in range(count)]
+    out_arr = (VP * count)(*[o.ptr for o in outs])
+    w_arr = (VP * count)(*[w.ptr for w in wd])
+    G.B.check(L.lcu_gemm_f16_nt_multi(out_arr, xd.ptr, w_arr, count, M, K, N, 0.0, None))
+    for g in range(count):
+        got = G.host(outs[g], (M, N))
+        assert G.max_abs_rel(got, sep[g]) <= TOL and G.ulp_mismatch(got, sep[g]) < 0.05, g
+        assert G.max_abs_rel(got, O.matmul_nt(x, ws[g])) <= TOL, g
+    if K % 128 == 0:
+        q = [O.quantize_absmax_u8(w, 128) for w in ws]
+        cd = [G.dev_keep(c) for c, _ in q]
+        sd = [G.dev_keep(sc) for _, sc in q]
+        sep = [G.gemm_u8(x, c, sc, 128) for c, sc in q]
+        c_arr = (VP * count)(*[c.ptr for c in cd])
+        s_arr = (VP * count)(*[sc.ptr for sc in sd])
+        G.B.check(L.lcu_gemm_f16u8_nt_multi(out_arr, xd.ptr, c_arr, s_arr, count, M, K, N, 128, 0.0, None))
+        for g in range(count):
+            got = G.host(outs[g], (M, N))
+            assert G.max_abs_rel(got, sep[g]) <= TOL and G.ulp_mismatch(got, sep[g]) < 0.05, g
+            assert G.max_abs_rel(got, O.matmul_nt_u8(x, q[g][0], q[g][1], 128)) <= TOL, g
+    assert L.lcu_gemm_f16_nt_multi(out_arr, xd.ptr, w_arr, 4, M, K, N, 0.0, None) == -2
+    G.release()
+
+
 def test_gemm_rejects_bad_shapes(gpu):
     G = gpu
     a = G.dev(np.zeros((4, 12), dtype=np.float16))

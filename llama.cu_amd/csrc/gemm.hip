@@ -897,7 +897,26 @@ int dispatch_gemm(operands_t op, const half_t* A, int M, int K, int N, int block
   // with two groups of four wavefronts splitting the K stage, because then the grid cannot give a
   // compute unit a second workgroup (M = 512, N = 4096: 35 us against 41 us, K = 11008: 100 us
   // against 135 us with the register-staged kernel).
-  // Several matrices of one shape (op.n_mats > 1) count as one product with n_mats * N columns.
+  // Several matrices of one shape (op.n_mats > 1) count as one product with n_mats * N columns --
+  // unless each of them already fills the chip with 256x128 tiles and fusing saves no round of
+  // workgroups (W1 + W3 at M = 512, N = 11008: 344 tiles take two rounds either way, and the fused
+  // launch measured 132 us against 2 x 63 us).
+  if (op.n_mats > 1 && M > 64 && K % 128 == 0) {
+    device_state* ds = current_device_state();
+    const long cus = ds && ds->compute_units > 0 ? ds->compute_units : 256;
+    const long per = (long)((M + 255) / 256) * ((N + 127) / 128);
+    if (per >= 160 && (per * op.n_mats + cus - 1) / cus >= op.n_mats * ((per + cus - 1) / cus)) {
+      for (int g = 0; g < op.n_mats; ++g) {
+        const operands_t one = single_matrix(g == 0 ? op.out : op.more.out[g - 1], g == 0 ? op.W : op.more.W[g - 1],
+                                             g == 0 ? op.S : op.more.S[g - 1]);
+        const int rc = dispatch_gemm<U8>(one, A, M, K, N, block, beta, st);
+        if (rc != LCU_OK) {
+          return rc;
+        }
+      }
+      return LCU_OK;
+    }
+  }
   const long nm = op.n_mats;
   const long tiles128 = (long)((M + 127) / 128) * ((N + 127) / 128) * nm;
   const long tiles64 = (long)((M + 127) / 128) * ((N + 63) / 64) * nm;

@@ -316,6 +316,12 @@ def test_silu_mul(gpu):
     ref = O.silu_mul(a, b)
     assert G.max_abs_rel(got, ref) <= TOL
     assert G.ulp_mismatch(got, ref) < 0.01
+    # ragged length (the last thread's eight elements are cut) and buffers off the 16-byte grid
+    for n2, off in ((2051, 0), (1000, 3)):
+        ad, bd, od = G.dev_keep(a[:n2 + off]), G.dev_keep(b[:n2 + off]), G.empty((n2 + off,))
+        G.B.check(G.L().lcu_silu_mul(od.ptr + 2 * off, ad.ptr + 2 * off, bd.ptr + 2 * off, n2, None))
+        got2 = G.host(od, (n2 + off,))[off:]
+        assert (got2.view(np.uint16) == got[off:n2 + off].view(np.uint16)).all()
     G.release()
 
 

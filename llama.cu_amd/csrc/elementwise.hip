@@ -209,6 +209,93 @@ __global__ __launch_bounds__(1024) void softmax_argmax_kernel(half_t* __restrict
   index += blockIdx.x;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int n8 = n / 8;
+  if (n % 8 == 0 && n8 <= 4 * 1024) {
+    // every vocabulary of the model family (n <= 32768): the row is read once and each element's
+    // x / temp, then its exponential, stays in registers -- the same operations in the same order
+    // as the general path below, which reads the row three times and takes each exponential twice
+    float t[4][8];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int c = tid + j * 1024;
+      const half8_t v = c < n8 ? *reinterpret_cast<const half8_t*>(logits + (size_t)c * 8) : (half8_t)(0.0f);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) t[j][e] = c < n8 ? (float)v[e] / temp : -INFINITY;
+    }
+    float m = -INFINITY;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) m = fmaxf(m, t[j][e]);
+    }
+    m = wave_max(m);
+    if (lane == 0) sred[wave] = m;
+    __syncthreads();
+    m = sred[0];
+#pragma unroll
+    for (int w = 1; w < 16; ++w) m = fmaxf(m, sred[w]);
+    __syncthreads();
+    float s = 0.0f;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      if (tid + j * 1024 < n8) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          t[j][e] = expf(t[j][e] - m);
+          s += t[j][e];
+        }
+      }
+    }
+    s = wave_sum(s);
+    if (lane == 0) sred[wave] = s;
+    __syncthreads();
+    float total = 0.0f;
+#pragma unroll
+    for (int w = 0; w < 16; ++w) total += sred[w];
+    __syncthreads();
+    float best = -INFINITY;
+    int idx = 0x7fffffff;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int c = tid + j * 1024;
+      if (c < n8) {
+        half8_t p;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          p[e] = round_f16(t[j][e] / total);
+          const float f = (float)p[e];
+          if (f > best) {  // ascending index within a thread: strict > keeps the first maximum
+            best = f;
+            idx = c * 8 + e;
+          }
+        }
+        *reinterpret_cast<half8_t*>(probs + (size_t)c * 8) = p;
+      }
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+      const float ob = __shfl_xor(best, off, WAVE);
+      const int oi = __shfl_xor(idx, off, WAVE);
+      if (ob > best || (ob == best && oi < idx)) {
+        best = ob;
+        idx = oi;
+      }
+    }
+    if (lane == 0) {
+      sred[wave] = best;
+      sidx[wave] = idx;
+    }
+    __syncthreads();
+    if (tid == 0) {
+      for (int w = 1; w < 16; ++w) {
+        if (sred[w] > best || (sred[w] == best && sidx[w] < idx)) {
+          best = sred[w];
+          idx = sidx[w];
+        }
+      }
+      *index = idx == 0x7fffffff ? 0 : idx;
+    }
+    return;
+  }
   float m = -INFINITY;
   for (int c = tid; c < n8; c += 1024) {
     const half8_t v = *reinterpret_cast<const half8_t*>(logits + (size_t)c * 8);

@@ -304,6 +304,7 @@ def main():
     ap.add_argument("--workload", default="llama7b_fp16", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip the per-shape GEMV / GEMM legs")
+    ap.add_argument("--no-batched", action="store_true", help="skip the batched-decode leg of the extra figures")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run one 256 MiB device-to-device copy: a copy kernel of known size, against which "
                          "rocprofv3 FETCH_SIZE / WRITE_SIZE readings of the other kernels are scaled")
@@ -324,7 +325,7 @@ def main():
                  decode_hbm_gb_s=round(dec["bytes_per_token"] / dec["ms_per_step"] / 1e6, 1),
                  decode_frac_of_hbm_roofline=round(dec["bytes_per_token"] / dec["ms_per_step"] / 1e6 / HBM_PEAK_GBS, 3))
     ctx.close()
-    if not args.no_extra:
+    if not args.no_extra and not args.no_batched:
         extra["batched_decode"] = batched_leg(P, model, cfg)
     model.close()
     if args.copy_calibration:

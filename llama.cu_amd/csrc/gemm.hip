@@ -441,6 +441,7 @@ __global__ __launch_bounds__(64 * WM * WN * KS, WM * WN * KS <= 4 ? 2 : 1) void 
   // stage 0, and where the two fp16 chunks of a dequantised chunk go in the W tile
   int d_scale[DC];
   uint32_t d_src[DC], d_dst0[DC], d_dst1[DC];
+  const bool hi_first = (tid >> 2) & 1;
   const int nblk = U8 ? K / block : 0;
   if constexpr (U8) {
 #pragma unroll
@@ -451,6 +452,15 @@ __global__ __launch_bounds__(64 * WM * WN * KS, WM * WN * KS <= 4 ? 2 : 1) void 
       d_src[i] = (uint32_t)c * 16;
       d_dst0[i] = (uint32_t)row * ROWB + (uint32_t)(((2 * kc) ^ f) * 16);
       d_dst1[i] = (uint32_t)row * ROWB + (uint32_t)(((2 * kc + 1) ^ f) * 16);
+      // LDS stores see 32 banks (128 bytes): eight consecutive lanes must land on eight different
+      // chunk positions modulo 8.  Four lanes share a row (or half a row) and would all write even
+      // positions with their first store; so every second group of four lanes writes its odd chunk
+      // first (8 conflict cycles per store instruction otherwise).
+      if (hi_first) {
+        const uint32_t t0 = d_dst0[i];
+        d_dst0[i] = d_dst1[i];
+        d_dst1[i] = t0;
+      }
     }
   }
   // A request is written as inline assembly (M0 = LDS address of the wavefront's 1 KB, then the
@@ -532,8 +542,8 @@ __global__ __launch_bounds__(64 * WM * WN * KS, WM * WN * KS <= 4 ? 2 : 1) void 
       const half8_t lo = {d[0].x, d[0].y, d[1].x, d[1].y, d[2].x, d[2].y, d[3].x, d[3].y};
       const half8_t hi = {d[4].x, d[4].y, d[5].x, d[5].y, d[6].x, d[6].y, d[7].x, d[7].y};
       unsigned char* tile = gemm_lds + B_BASE + bslot * B_STRIDE;
-      *reinterpret_cast<half8_t*>(tile + d_dst0[i]) = lo;
-      *reinterpret_cast<half8_t*>(tile + d_dst1[i]) = hi;
+      *reinterpret_cast<half8_t*>(tile + d_dst0[i]) = hi_first ? hi : lo;
+      *reinterpret_cast<half8_t*>(tile + d_dst1[i]) = hi_first ? lo : hi;
     }
   };
 

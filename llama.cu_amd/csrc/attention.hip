@@ -298,6 +298,12 @@ constexpr int QLD = HD + 8;    // LDS row stride (halves) of the Q and K tiles
 constexpr int MAX_T_PREFILL = 2048;
 
 // BR: query rows per workgroup (16 or 32)
+// LDS row of position p of a V chunk (a permutation inside every block of 32 positions)
+__device__ __forceinline__ int v_row(int p) {
+  const int e = p & 7, g = (p >> 3) & 3;
+  return (p & ~31) + 4 * g + (e & 3) + 16 * (e >> 2);
+}
+
 template <int BR>
 __global__ __launch_bounds__(256) void prefill_attention_kernel(half_t* __restrict__ out, const half_t* __restrict__ q,
                                                                 const half_t* __restrict__ k, const half_t* __restrict__ v,
@@ -345,11 +351,15 @@ __global__ __launch_bounds__(256) void prefill_attention_kernel(half_t* __restri
       reg[i] = *reinterpret_cast<const half8_t*>(src + (size_t)gp * dim + h * HD + (c & 15) * 8);
     }
   };
+  // V rows are stored in a permuted order (see the gather below); K rows in their own
+  bool permute_rows = false;
   auto store_chunk = [&](const half8_t (&reg)[CH]) {
 #pragma unroll
     for (int i = 0; i < CH; ++i) {
       const int c = tid + i * 256;
-      *reinterpret_cast<half8_t*>(&KVs[(c >> 4) * QLD + (c & 15) * 8]) = reg[i];
+      const int p = c >> 4;
+      const int row = permute_rows ? v_row(p) : p;
+      *reinterpret_cast<half8_t*>(&KVs[row * QLD + (c & 15) * 8]) = reg[i];
     }
   };
 
@@ -416,17 +426,29 @@ __global__ __launch_bounds__(256) void prefill_attention_kernel(half_t* __restri
   // expf the softmax was the longest phase of the kernel.
   constexpr float LOG2E = 1.4426950408889634f;
   for (int rr = 0; rr < BR / 4; ++rr) {
-    half_t* srow = Ss + (wave * (BR / 4) + rr) * SLD;
+    // two neighbouring scores per lane and access (4 bytes: whole LDS words)
+    half2_t* srow = reinterpret_cast<half2_t*>(Ss + (wave * (BR / 4) + rr) * SLD);
+    const int pairs = Tc / 2;
     float m = -INFINITY;
-    for (int i = lane; i < Tc; i += WAVE) m = fmaxf(m, (float)srow[i]);
+    for (int i = lane; i < pairs; i += WAVE) {
+      const half2_t v = srow[i];
+      m = fmaxf(m, fmaxf((float)v.x, (float)v.y));
+    }
     m = wave_max(m);
     const float m2 = m * LOG2E;
     float s = 0.0f;
-    for (int i = lane; i < Tc; i += WAVE) s += __builtin_amdgcn_exp2f(fmaf((float)srow[i], LOG2E, -m2));
+    for (int i = lane; i < pairs; i += WAVE) {
+      const half2_t v = srow[i];
+      s += __builtin_amdgcn_exp2f(fmaf((float)v.x, LOG2E, -m2)) + __builtin_amdgcn_exp2f(fmaf((float)v.y, LOG2E, -m2));
+    }
     s = wave_sum(s);
     const float inv = __builtin_amdgcn_rcpf(s);
-    for (int i = lane; i < Tc; i += WAVE) {
-      srow[i] = round_f16(__builtin_amdgcn_exp2f(fmaf((float)srow[i], LOG2E, -m2)) * inv);
+    for (int i = lane; i < pairs; i += WAVE) {
+      const half2_t v = srow[i];
+      half2_t p;
+      p.x = round_f16(__builtin_amdgcn_exp2f(fmaf((float)v.x, LOG2E, -m2)) * inv);
+      p.y = round_f16(__builtin_amdgcn_exp2f(fmaf((float)v.y, LOG2E, -m2)) * inv);
+      srow[i] = p;
     }
   }
 
@@ -439,7 +461,12 @@ __global__ __launch_bounds__(256) void prefill_attention_kernel(half_t* __restri
   }
   // V chunks stay row-major in LDS, KVs[pos][d] (16-byte stores without bank conflicts); the
   // matrix instruction wants 8 consecutive positions of one output column per lane, which are
-  // gathered with 2-byte reads: the 16 lanes of a fragment row group read 16 neighbouring columns.
+  // gathered with 2-byte reads: the 16 lanes of a fragment row group read 16 neighbouring columns
+  // (32 bytes), the four groups rows 8 positions apart.  A row is 272 bytes, so 8 rows apart is
+  // 128 bytes modulo the 256 bytes of the banks and groups 0 and 2 (1 and 3) would meet in the same
+  // banks; v_row() places position 8g + e of a 32-row block at row 4g + e % 4 + 16 (e / 4), which
+  // puts the four groups 64 bytes apart.
+  permute_rows = true;
   for_chunks(v, [&](int c0) {
 #pragma unroll
     for (int ks = 0; ks < CW; ks += 32) {
@@ -448,9 +475,9 @@ __global__ __launch_bounds__(256) void prefill_attention_kernel(half_t* __restri
       for (int i = 0; i < RT; ++i) fa[i] = *reinterpret_cast<const half8_t*>(&Ss[(i * 16 + frow) * SLD + c0 + ks + fk]);
 #pragma unroll
       for (int j = 0; j < 2; ++j) {
-        const half_t* vcol = &KVs[(ks + fk) * QLD + wave * 32 + j * 16 + frow];
+        const half_t* vcol = &KVs[(ks + fk / 2) * QLD + wave * 32 + j * 16 + frow];  // v_row(ks + fk + e) below
 #pragma unroll
-        for (int e = 0; e < 8; ++e) fb[j][e] = vcol[e * QLD];
+        for (int e = 0; e < 8; ++e) fb[j][e] = vcol[((e & 3) + 16 * (e >> 2)) * QLD];
       }
 #pragma unroll
       for (int i = 0; i < RT; ++i) {

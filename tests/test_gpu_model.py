@@ -186,6 +186,35 @@ def test_batched_decode_vs_oracle(gpu, q_type):
     gm.close()
 
 
+def test_batched_decode_with_a_long_and_a_short_sequence(gpu):
+    """One sequence beyond 1024 cached rows (where a single context switches its attention form and the batch
+    raises its bound), one at the start: both follow their own single-sequence contexts."""
+    G = gpu
+    gm = G.P.Model(**SMALL, seed=17, weight_std=0.05)
+    rng = np.random.default_rng(3)
+    prompts = [rng.integers(0, SMALL["n_vocab"], n).astype(np.int16) for n in (1021, 5)]
+    singles = [G.P.Context(gm, context_len=2048, temperature=0.8) for _ in prompts]
+    bc = G.P.BatchContext(gm, 2, context_len=2048, temperature=0.8)
+    last = []
+    for b, pr in enumerate(prompts):
+        t = singles[b].next_token(pr)
+        assert bc.next_token(b, pr) == t
+        last.append(t)
+    for k in range(6):   # positions 1021..1026 and 5..10: the bound changes from 1024 to 2048 on the way
+        want = [c.next_token([t]) for c, t in zip(singles, last)]
+        got = bc.next_tokens(last)
+        logits = bc.logits()
+        for b in range(2):
+            ref = singles[b].logits()
+            assert G.max_abs_rel(logits[b], ref) <= TOL, (k, b)
+            lo = np.sort(ref.astype(np.float32))
+            if lo[-1] - lo[-2] > 0.05:
+                assert got[b] == want[b], (k, b)
+        last = want
+    for o in singles + [bc, gm]:
+        o.close()
+
+
 def test_context_api_behaviour(gpu):
     G = gpu
     gm = G.P.Model(**TINY, seed=1)

@@ -169,6 +169,22 @@ int lcu_rope_store_batch(void* q_dev, const void* k_new_dev, const void* v_new_d
 int lcu_attention_decode_batch(void* out_dev, const void* q_dev, const void* k_cache_ptrs_dev,
                                const void* v_cache_ptrs_dev, const void* pos_dev, int n_seq, int max_T, int dim,
                                int n_heads, void* stream);
+/* The products of a batched step fused with what follows them (for 2..64 sequences the partial sums
+ * of the split-K product are added up by the kernel that goes on with them; any other shape runs
+ * the separate operators above).  w_dev / scales_dev: host arrays of device pointers (scales NULL
+ * and block 0 for fp16 weights); *_tmp_dev: [n_seq][dim] / [n_seq][ffn] fp16 scratch.
+ *   lcu_batch_qkv: Wq, Wk, Wv products of lhs [n_seq][dim], then lcu_rope_store_batch (1144-1156)
+ *   lcu_batch_ffn_up: W1, W3 products, then fp16(silu(w1) * w3) (1180-1183)
+ *   lcu_batch_proj_norm: x += lhs [n_seq][K] * W^T (1174 / 1185), then norm_out = rms_norm(x) with
+ *     norm_w (1176, or 1129 of the next layer, or 1191) */
+int lcu_batch_qkv(void* q_out_dev, void* k_tmp_dev, void* v_tmp_dev, const void* lhs_dev, const void* const* w_dev,
+                  const void* const* scales_dev, int block, int n_seq, int dim, int n_heads,
+                  const void* k_cache_ptrs_dev, const void* v_cache_ptrs_dev, const void* pos_dev,
+                  const void* table_dev, int table_positions, void* stream);
+int lcu_batch_ffn_up(void* out_dev, void* w1_tmp_dev, void* w3_tmp_dev, const void* lhs_dev, const void* const* w_dev,
+                     const void* const* scales_dev, int block, int n_seq, int dim, int ffn, void* stream);
+int lcu_batch_proj_norm(void* x_dev, void* norm_out_dev, const void* lhs_dev, const void* w_dev, const void* scales_dev,
+                        int block, int n_seq, int K, int dim, const void* norm_w_dev, float eps, void* stream);
 /* lcu_softmax_argmax on `rows` rows of n logits (n a multiple of 8): probabilities [rows][n],
  * one int32 index per row */
 int lcu_softmax_argmax_rows(void* probs_dev, void* out_index_dev, const void* logits_dev, int rows, int n, float temp,

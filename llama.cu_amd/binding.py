@@ -64,6 +64,9 @@ SIGNATURES = {
     "lcu_rope_store_batch": (i32, [vp, vp, vp, vp, vp, vp, i32, i32, i32, vp, i32, vp]),
     "lcu_attention_decode_batch": (i32, [vp, vp, vp, vp, vp, i32, i32, i32, i32, vp]),
     "lcu_softmax_argmax_rows": (i32, [vp, vp, vp, i32, i32, f32, vp]),
+    "lcu_batch_qkv": (i32, [vp, vp, vp, vp, vp, vp, i32, i32, i32, i32, vp, vp, vp, vp, i32, vp]),
+    "lcu_batch_ffn_up": (i32, [vp, vp, vp, vp, vp, vp, i32, i32, i32, i32, vp]),
+    "lcu_batch_proj_norm": (i32, [vp, vp, vp, vp, vp, i32, i32, i32, i32, vp, f32, vp]),
     "lcu_attention": (i32, [vp, vp, vp, vp, i32, i32, i32, i32, i32, vp]),
     "lcu_decode_qkv": (i32, [vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, i32, i32, i32, i32, vp, f32, vp, i32, vp]),
     "lcu_attention_decode": (i32, [vp, vp, vp, vp, vp, i32, i32, i32, vp]),

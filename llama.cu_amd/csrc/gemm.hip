@@ -810,9 +810,15 @@ int launch_dl(operands_t op, const half_t* A, int M, int K, int N, int block, fl
 // BM x 128 tiles with four wavefronts, the K stages split over enough workgroups to give every
 // compute unit one, fp32 partial sums in the per-device workspace, then splitk_reduce_kernel.
 // Returns LCU_OK with *done = false when the shape does not suit it.
+// where a split-K launch left its partial sums: part[matrix][split][M][N] fp32
+struct partial_sums_t {
+  const float* part;
+  int splits;
+};
+
 template <int BM, bool U8>
 int launch_skinny(operands_t op, const half_t* A, int M, int K, int N, int block, float beta, hipStream_t st,
-                  bool* done) {
+                  bool* done, partial_sums_t* leave = nullptr) {
   // a ring of six stages and 128-wide stages with eight wavefronts measured no faster
   constexpr int BN = 128, WM = 1, WN = 4, KS = 1, NS = 3;
   constexpr int ROWB = BK * KS * 2;
@@ -854,11 +860,175 @@ int launch_skinny(operands_t op, const half_t* A, int M, int K, int N, int block
   kernel<<<tiles_m * tiles_n * splits, 256 * KS, lds, st>>>(op.out, A, op.W, op.S, M, K, N, block, beta, tiles_m, tiles_n,
                                                             part, splits, op.more);
   LCU_LAUNCH_CHECK();
-  splitk_reduce_kernel<<<dim3((unsigned)((mn + 1023) / 1024), op.n_mats), 256, 0, st>>>(
-      op.out, op.more.out[0], op.more.out[1], part, mn, splits, beta);
-  LCU_LAUNCH_CHECK();
+  if (leave) {  // the caller's own kernel adds the partial sums up (fused with what follows the product)
+    leave->part = part;
+    leave->splits = splits;
+  } else {
+    splitk_reduce_kernel<<<dim3((unsigned)((mn + 1023) / 1024), op.n_mats), 256, 0, st>>>(
+        op.out, op.more.out[0], op.more.out[1], part, mn, splits, beta);
+    LCU_LAUNCH_CHECK();
+  }
   *done = true;
   return LCU_OK;
+}
+
+// the split-K product of a few rows with its partial sums left in the workspace; *done = false when
+// the shape does not take that path (nothing has been launched then)
+template <bool U8>
+int skinny_partial(operands_t op, const half_t* A, int M, int K, int N, int block, hipStream_t st, bool* done,
+                   partial_sums_t* res) {
+  *done = false;
+  if (K % 128 != 0 || M > 64 || M < 1) {
+    return LCU_OK;
+  }
+  if constexpr (U8) {
+    return launch_skinny<32, true>(op, A, M, K, N, block, 0.0f, st, done, res);
+  } else {
+    return M <= 32 ? launch_skinny<32, false>(op, A, M, K, N, block, 0.0f, st, done, res)
+                   : launch_skinny<64, false>(op, A, M, K, N, block, 0.0f, st, done, res);
+  }
+}
+
+// ---- kernels that add the partial sums up and go on with what follows the product in a batched
+// decode step (llama_cu.cu:1144-1156, 1174-1176, 1180-1185), one row per sequence ----
+
+__device__ __forceinline__ float2 sum_pair(const float* __restrict__ part, size_t at, size_t mn, int splits) {
+  float2 v = *reinterpret_cast<const float2*>(part + at);
+  for (int s = 1; s < splits; ++s) {
+    const float2 w = *reinterpret_cast<const float2*>(part + (size_t)s * mn + at);
+    v.x += w.x;
+    v.y += w.y;
+  }
+  return v;
+}
+
+// Wq, Wk, Wv products -> fp16 -> rotary of q (to q_out) and k at pos[b]; rotated k and v into row
+// pos[b] of sequence b's caches (what splitk_reduce_kernel + rope_store_batch_kernel do)
+__global__ __launch_bounds__(256) void reduce_rope_store_kernel(half_t* __restrict__ q_out, const float* __restrict__ part,
+                                                                int splits, int n_seq, int dim,
+                                                                half_t* const* __restrict__ k_ptrs,
+                                                                half_t* const* __restrict__ v_ptrs,
+                                                                const int* __restrict__ pos_dev, int head_dim,
+                                                                const float2* __restrict__ table, int max_pos) {
+  const int pair = blockIdx.x * 256 + threadIdx.x;
+  const int b = blockIdx.y;
+  if (pair * 2 >= dim) return;
+  const int c = pair * 2;
+  const size_t mn = (size_t)n_seq * dim, at = (size_t)b * dim + c;
+  const int pos = min(max(pos_dev[b], 0), max_pos);
+  const float2 cs = table[(size_t)pos * (head_dim / 2) + (c % head_dim) / 2];
+  const float2 qf = sum_pair(part, at, mn, splits);
+  const float2 kf = sum_pair(part + (size_t)splits * mn, at, mn, splits);
+  const float2 vf = sum_pair(part + (size_t)2 * splits * mn, at, mn, splits);
+  // the products are rounded to fp16 before the rotary reads them (1144-1153)
+  const float qr = (float)round_f16(qf.x), qi = (float)round_f16(qf.y);
+  const float kr = (float)round_f16(kf.x), ki = (float)round_f16(kf.y);
+  half2_t w;
+  w.x = round_f16(fmaf(qr, cs.x, -(qi * cs.y)));
+  w.y = round_f16(fmaf(qr, cs.y, qi * cs.x));
+  *reinterpret_cast<half2_t*>(q_out + at) = w;
+  const size_t dst = (size_t)pos * dim + c;
+  w.x = round_f16(fmaf(kr, cs.x, -(ki * cs.y)));
+  w.y = round_f16(fmaf(kr, cs.y, ki * cs.x));
+  *reinterpret_cast<half2_t*>(k_ptrs[b] + dst) = w;
+  w.x = round_f16(vf.x);
+  w.y = round_f16(vf.y);
+  *reinterpret_cast<half2_t*>(v_ptrs[b] + dst) = w;
+}
+
+// W1, W3 products -> fp16 each -> fp16(silu(w1) * w3)  (1180-1183, 533-539)
+__global__ __launch_bounds__(256) void reduce_silu_kernel(half_t* __restrict__ out, const float* __restrict__ part,
+                                                          int splits, size_t mn) {
+  const size_t i = ((size_t)blockIdx.x * 256 + threadIdx.x) * 2;
+  if (i >= mn) return;
+  const float2 a = sum_pair(part, i, mn, splits);
+  const float2 g = sum_pair(part + (size_t)splits * mn, i, mn, splits);
+  const float v0 = (float)round_f16(a.x), v1 = (float)round_f16(a.y);
+  half2_t w;
+  w.x = round_f16(v0 / (1.0f + expf(-v0)) * (float)round_f16(g.x));
+  w.y = round_f16(v1 / (1.0f + expf(-v1)) * (float)round_f16(g.y));
+  *reinterpret_cast<half2_t*>(out + i) = w;
+}
+
+// x += product (one rounding of the fp32 sum, 1174 / 1185), then rms_norm of the new row with the
+// next norm's weights (1176 / 1129 of the next layer / 1191).  One 1024-thread workgroup per row
+// (up to 8192 columns: four pairs per thread, every partial sum requested before the first is
+// used -- the launch is a handful of workgroups and nothing but latency); the norm as in
+// rmsnorm_kernel, its sum of squares taken by the first 256 threads in the reference's association.
+constexpr int RN_THREADS = 1024, RN_PAIRS = 4;
+__global__ __launch_bounds__(RN_THREADS) void reduce_residual_norm_kernel(half_t* __restrict__ x,
+                                                                          half_t* __restrict__ norm_out,
+                                                                          const float* __restrict__ part, int splits,
+                                                                          int n_seq, int cols,
+                                                                          const half_t* __restrict__ norm_w, float eps) {
+  extern __shared__ half_t row_lds[];
+  __shared__ float red[8];
+  const int b = blockIdx.x, tid = threadIdx.x;
+  const size_t mn = (size_t)n_seq * cols;
+  half_t* xr = x + (size_t)b * cols;
+  float2 acc[RN_PAIRS];
+  half2_t old[RN_PAIRS], wv[RN_PAIRS];
+#pragma unroll
+  for (int j = 0; j < RN_PAIRS; ++j) {
+    const int c = min((tid + j * RN_THREADS) * 2, cols - 2);
+    acc[j] = *reinterpret_cast<const float2*>(part + (size_t)b * cols + c);
+    old[j] = *reinterpret_cast<const half2_t*>(xr + c);
+    wv[j] = *reinterpret_cast<const half2_t*>(norm_w + c);
+  }
+  for (int s = 1; s < splits; ++s) {
+#pragma unroll
+    for (int j = 0; j < RN_PAIRS; ++j) {
+      const int c = min((tid + j * RN_THREADS) * 2, cols - 2);
+      const float2 w = *reinterpret_cast<const float2*>(part + (size_t)s * mn + (size_t)b * cols + c);
+      acc[j].x += w.x;
+      acc[j].y += w.y;
+    }
+  }
+  half2_t val[RN_PAIRS];
+#pragma unroll
+  for (int j = 0; j < RN_PAIRS; ++j) {
+    const int c = (tid + j * RN_THREADS) * 2;
+    val[j].x = round_f16(fmaf(1.0f, (float)old[j].x, acc[j].x));
+    val[j].y = round_f16(fmaf(1.0f, (float)old[j].y, acc[j].y));
+    if (c < cols) {
+      *reinterpret_cast<half2_t*>(xr + c) = val[j];
+      *reinterpret_cast<half2_t*>(row_lds + c) = val[j];
+    }
+  }
+  __syncthreads();
+  float s = 0.0f;
+  if (tid < 256) {
+    for (int i = tid; i < cols; i += 256) {
+      const float v = (float)row_lds[i];
+      s = fmaf(v, v, s);
+    }
+  }
+  // block256_sum_ref_order for the first 256 threads of a larger workgroup
+#pragma unroll
+  for (int off = 16; off > 0; off >>= 1) {
+    s += __shfl_xor(s, off, WAVE);
+  }
+  if (tid < 256 && (tid & 31) == 0) {
+    red[tid >> 5] = s;
+  }
+  __syncthreads();
+  float total = red[tid & 7];
+#pragma unroll
+  for (int off = 4; off > 0; off >>= 1) {
+    total += __shfl_xor(total, off, WAVE);
+  }
+  const float rms_inv = 1.0f / sqrtf(total / (float)cols + eps);
+  half_t* y = norm_out + (size_t)b * cols;
+#pragma unroll
+  for (int j = 0; j < RN_PAIRS; ++j) {
+    const int c = (tid + j * RN_THREADS) * 2;
+    if (c < cols) {
+      half2_t r;
+      r.x = round_f16((float)wv[j].x * (float)round_f16((float)val[j].x * rms_inv));
+      r.y = round_f16((float)wv[j].y * (float)round_f16((float)val[j].y * rms_inv));
+      *reinterpret_cast<half2_t*>(y + c) = r;
+    }
+  }
 }
 
 template <int BM, int BN, int KS>
@@ -1067,6 +1237,118 @@ int lcu_gemm_f16u8_nt_multi(void* const* out_dev, const void* lhs_dev, const voi
     op.more.S[g - 1] = (const half_t*)scales_dev[g];
   }
   return dispatch_gemm<true>(op, (const half_t*)lhs_dev, M, K, N, block, beta, as_stream(stream));
+}
+
+// ---- fused steps of a batched decode (one row per sequence) ----
+
+static operands_t make_operands(void* const* outs, const void* const* values, const void* const* scales, int count) {
+  operands_t op = single_matrix((half_t*)(outs ? outs[0] : nullptr), values[0], (const half_t*)(scales ? scales[0] : nullptr));
+  op.n_mats = count;
+  for (int g = 1; g < count; ++g) {
+    op.more.out[g - 1] = (half_t*)(outs ? outs[g] : nullptr);
+    op.more.W[g - 1] = values[g];
+    op.more.S[g - 1] = (const half_t*)(scales ? scales[g] : nullptr);
+  }
+  return op;
+}
+
+int lcu_batch_qkv(void* q_out_dev, void* k_tmp_dev, void* v_tmp_dev, const void* lhs_dev, const void* const* w_dev,
+                  const void* const* scales_dev, int block, int n_seq, int dim, int n_heads,
+                  const void* k_cache_ptrs_dev, const void* v_cache_ptrs_dev, const void* pos_dev,
+                  const void* table_dev, int table_positions, void* stream) {
+  LCU_REQUIRE(q_out_dev && k_tmp_dev && v_tmp_dev && lhs_dev && w_dev && w_dev[0] && w_dev[1] && w_dev[2] &&
+                  k_cache_ptrs_dev && v_cache_ptrs_dev && pos_dev && table_dev,
+              "lcu_batch_qkv: null pointer");
+  LCU_REQUIRE(n_seq >= 0 && dim > 0 && n_heads > 0 && dim % n_heads == 0 && (dim / n_heads) % 2 == 0 && dim % 16 == 0 &&
+                  table_positions > 0,
+              "lcu_batch_qkv: bad shape n_seq %d dim %d heads %d", n_seq, dim, n_heads);
+  LCU_REQUIRE(block == 0 || (scales_dev && scales_dev[0] && scales_dev[1] && scales_dev[2] && block % 16 == 0 &&
+                             dim % block == 0),
+              "lcu_batch_qkv: quantised weights need scales and a block dividing dim");
+  if (n_seq == 0) return LCU_OK;
+  hipStream_t st = as_stream(stream);
+  void* const outs[3] = {q_out_dev, k_tmp_dev, v_tmp_dev};
+  bool done = false;
+  partial_sums_t ps{};
+  if (n_seq > 1) {
+    const operands_t op = make_operands(outs, w_dev, block ? scales_dev : nullptr, 3);
+    const int rc = block ? skinny_partial<true>(op, (const half_t*)lhs_dev, n_seq, dim, dim, block, st, &done, &ps)
+                         : skinny_partial<false>(op, (const half_t*)lhs_dev, n_seq, dim, dim, 0, st, &done, &ps);
+    if (rc != LCU_OK) return rc;
+  }
+  if (done) {
+    reduce_rope_store_kernel<<<dim3((dim / 2 + 255) / 256, n_seq), 256, 0, st>>>(
+        (half_t*)q_out_dev, ps.part, ps.splits, n_seq, dim, (half_t* const*)k_cache_ptrs_dev,
+        (half_t* const*)v_cache_ptrs_dev, (const int*)pos_dev, dim / n_heads, (const float2*)table_dev,
+        table_positions - 1);
+    LCU_LAUNCH_CHECK();
+    return LCU_OK;
+  }
+  // any other shape: the three products, then rotary and cache append
+  const int rc = block ? lcu_gemm_f16u8_nt_multi(outs, lhs_dev, w_dev, scales_dev, 3, n_seq, dim, dim, block, 0.0f, stream)
+                       : lcu_gemm_f16_nt_multi(outs, lhs_dev, w_dev, 3, n_seq, dim, dim, 0.0f, stream);
+  if (rc != LCU_OK) return rc;
+  return lcu_rope_store_batch(q_out_dev, k_tmp_dev, v_tmp_dev, k_cache_ptrs_dev, v_cache_ptrs_dev, pos_dev, n_seq, dim,
+                              n_heads, table_dev, table_positions, stream);
+}
+
+int lcu_batch_ffn_up(void* out_dev, void* w1_tmp_dev, void* w3_tmp_dev, const void* lhs_dev, const void* const* w_dev,
+                     const void* const* scales_dev, int block, int n_seq, int dim, int ffn, void* stream) {
+  LCU_REQUIRE(out_dev && w1_tmp_dev && w3_tmp_dev && lhs_dev && w_dev && w_dev[0] && w_dev[1], "lcu_batch_ffn_up: null pointer");
+  LCU_REQUIRE(n_seq >= 0 && dim > 0 && ffn > 0 && dim % 16 == 0 && ffn % 2 == 0, "lcu_batch_ffn_up: bad shape n_seq %d dim %d ffn %d",
+              n_seq, dim, ffn);
+  LCU_REQUIRE(block == 0 || (scales_dev && scales_dev[0] && scales_dev[1] && block % 16 == 0 && dim % block == 0),
+              "lcu_batch_ffn_up: quantised weights need scales and a block dividing dim");
+  if (n_seq == 0) return LCU_OK;
+  hipStream_t st = as_stream(stream);
+  void* const outs[2] = {w1_tmp_dev, w3_tmp_dev};
+  bool done = false;
+  partial_sums_t ps{};
+  if (n_seq > 1) {
+    const operands_t op = make_operands(outs, w_dev, block ? scales_dev : nullptr, 2);
+    const int rc = block ? skinny_partial<true>(op, (const half_t*)lhs_dev, n_seq, dim, ffn, block, st, &done, &ps)
+                         : skinny_partial<false>(op, (const half_t*)lhs_dev, n_seq, dim, ffn, 0, st, &done, &ps);
+    if (rc != LCU_OK) return rc;
+  }
+  if (done) {
+    const size_t mn = (size_t)n_seq * ffn;
+    reduce_silu_kernel<<<(unsigned)((mn / 2 + 255) / 256), 256, 0, st>>>((half_t*)out_dev, ps.part, ps.splits, mn);
+    LCU_LAUNCH_CHECK();
+    return LCU_OK;
+  }
+  const int rc = block ? lcu_gemm_f16u8_nt_multi(outs, lhs_dev, w_dev, scales_dev, 2, n_seq, dim, ffn, block, 0.0f, stream)
+                       : lcu_gemm_f16_nt_multi(outs, lhs_dev, w_dev, 2, n_seq, dim, ffn, 0.0f, stream);
+  if (rc != LCU_OK) return rc;
+  return lcu_silu_mul(out_dev, w1_tmp_dev, w3_tmp_dev, (size_t)n_seq * ffn, stream);
+}
+
+int lcu_batch_proj_norm(void* x_dev, void* norm_out_dev, const void* lhs_dev, const void* w_dev, const void* scales_dev,
+                        int block, int n_seq, int K, int dim, const void* norm_w_dev, float eps, void* stream) {
+  LCU_REQUIRE(x_dev && norm_out_dev && lhs_dev && w_dev && norm_w_dev, "lcu_batch_proj_norm: null pointer");
+  LCU_REQUIRE(n_seq >= 0 && dim > 0 && K > 0 && K % 16 == 0 && dim % 2 == 0 && dim <= 24576,
+              "lcu_batch_proj_norm: bad shape n_seq %d K %d dim %d", n_seq, K, dim);
+  LCU_REQUIRE(block == 0 || (scales_dev && block % 16 == 0 && K % block == 0),
+              "lcu_batch_proj_norm: quantised weights need scales and a block dividing K");
+  if (n_seq == 0) return LCU_OK;
+  hipStream_t st = as_stream(stream);
+  bool done = false;
+  partial_sums_t ps{};
+  if (n_seq > 1 && dim <= RN_THREADS * RN_PAIRS * 2) {
+    const operands_t op = single_matrix((half_t*)x_dev, w_dev, (const half_t*)(block ? scales_dev : nullptr));
+    const int rc = block ? skinny_partial<true>(op, (const half_t*)lhs_dev, n_seq, K, dim, block, st, &done, &ps)
+                         : skinny_partial<false>(op, (const half_t*)lhs_dev, n_seq, K, dim, 0, st, &done, &ps);
+    if (rc != LCU_OK) return rc;
+  }
+  if (done) {
+    reduce_residual_norm_kernel<<<n_seq, RN_THREADS, (size_t)dim * 2, st>>>(
+        (half_t*)x_dev, (half_t*)norm_out_dev, ps.part, ps.splits, n_seq, dim, (const half_t*)norm_w_dev, eps);
+    LCU_LAUNCH_CHECK();
+    return LCU_OK;
+  }
+  const int rc = block ? lcu_gemm_f16u8_nt(x_dev, lhs_dev, w_dev, scales_dev, n_seq, K, dim, block, 1.0f, stream)
+                       : lcu_gemm_f16_nt(x_dev, lhs_dev, w_dev, n_seq, K, dim, 1.0f, stream);
+  if (rc != LCU_OK) return rc;
+  return lcu_rmsnorm(norm_out_dev, x_dev, norm_w_dev, n_seq, dim, eps, stream);
 }
 
 }  // extern "C"

@@ -154,22 +154,6 @@ struct llama_batch_context_impl final : public llama_batch_context {
     }
   }
 
-  void matmul_multi(void* const* outs, const void* lhs, weight_tensor const* const* ws, int count, int M) {
-    const void* values[3];
-    const void* scales[3];
-    for (int g = 0; g < count; ++g) {
-      values[g] = ws[g]->data.data();
-      scales[g] = ws[g]->scales.data();
-    }
-    weight_tensor const& w = *ws[0];
-    if (w.quantised) {
-      LCU_CHECK(lcu_gemm_f16u8_nt_multi(outs, lhs, values, scales, count, M, (int)w.cols, (int)w.rows, w.block, 0.0f,
-                                        stream_));
-    } else {
-      LCU_CHECK(lcu_gemm_f16_nt_multi(outs, lhs, values, count, M, (int)w.cols, (int)w.rows, 0.0f, stream_));
-    }
-  }
-
   void enqueue_step(int bound) {
     llama_params const& p = model_->params;
     const int B = (int)seqs_.size(), dim = p.dim, ffn = p.ffn_dim(), heads = p.n_heads, vocab = p.n_vocab;
@@ -183,28 +167,32 @@ struct llama_batch_context_impl final : public llama_batch_context {
     } else {
       LCU_CHECK(lcu_embed(x, ids, B, dim, model_->tok_embeddings.data.data(), vocab, stream_));
     }
-    for (size_t l = 0; l < model_->layers.size(); ++l) {
+    // Every product is fused with what follows it (lcu_batch_*): rotary + cache append after
+    // Wq/Wk/Wv, SiLU after W1/W3, the residual sum and the NEXT norm after Wo and W2 -- so the
+    // first norm stands alone and the last W2 carries the final norm.
+    LCU_CHECK(lcu_rmsnorm(t_norm_.data(), x, model_->layers[0].attn_norm.data(), B, dim, p.norm_eps, stream_));  // 1129
+    const size_t n_layers = model_->layers.size();
+    for (size_t l = 0; l < n_layers; ++l) {
       llama_layer const& L = model_->layers[l];
       const char* kp = (char*)t_cache_ptrs_.data() + (l * 2 + 0) * B * sizeof(void*);
       const char* vp = (char*)t_cache_ptrs_.data() + (l * 2 + 1) * B * sizeof(void*);
-      LCU_CHECK(lcu_rmsnorm(t_norm_.data(), x, L.attn_norm.data(), B, dim, p.norm_eps, stream_));         // 1129
-      void* const qkv_out[3] = {t_q_.data(), t_k_.data(), t_v_.data()};
-      weight_tensor const* const qkv_w[3] = {&L.wq, &L.wk, &L.wv};
-      matmul_multi(qkv_out, t_norm_.data(), qkv_w, 3, B);                                                  // 1144, 1150, 1156
-      LCU_CHECK(lcu_rope_store_batch(t_q_.data(), t_k_.data(), t_v_.data(), kp, vp, pos, B, dim, heads,
-                                     seqs_[0]->rope_table(), context_len_, stream_));                      // 1146, 1152
+      const void* const qkv_w[3] = {L.wq.data.data(), L.wk.data.data(), L.wv.data.data()};
+      const void* const qkv_s[3] = {L.wq.scales.data(), L.wk.scales.data(), L.wv.scales.data()};
+      LCU_CHECK(lcu_batch_qkv(t_q_.data(), t_k_.data(), t_v_.data(), t_norm_.data(), qkv_w, qkv_s, block, B, dim, heads,
+                              kp, vp, pos, seqs_[0]->rope_table(), context_len_, stream_));                // 1144-1156
       LCU_CHECK(lcu_attention_decode_batch(t_out_.data(), t_q_.data(), kp, vp, pos, B, bound, dim, heads,
                                            stream_));                                                      // 1161-1171
-      matmul(x, t_out_.data(), L.wo, B, 1.0f);                                                             // 1174
-      LCU_CHECK(lcu_rmsnorm(t_norm_.data(), x, L.ffn_norm.data(), B, dim, p.norm_eps, stream_));          // 1176
-      void* const up_out[2] = {t_w1_.data(), t_w3_.data()};
-      weight_tensor const* const up_w[2] = {&L.w1, &L.w3};
-      matmul_multi(up_out, t_norm_.data(), up_w, 2, B);                                                    // 1180, 1181
-      LCU_CHECK(lcu_silu_mul(t_silu_.data(), t_w1_.data(), t_w3_.data(), (size_t)B * ffn, stream_));      // 1183
-      matmul(x, t_silu_.data(), L.w2, B, 1.0f);                                                            // 1185
+      LCU_CHECK(lcu_batch_proj_norm(x, t_norm_.data(), t_out_.data(), L.wo.data.data(), L.wo.scales.data(), block, B,
+                                    dim, dim, L.ffn_norm.data(), p.norm_eps, stream_));                    // 1174, 1176
+      const void* const up_w[2] = {L.w1.data.data(), L.w3.data.data()};
+      const void* const up_s[2] = {L.w1.scales.data(), L.w3.scales.data()};
+      LCU_CHECK(lcu_batch_ffn_up(t_silu_.data(), t_w1_.data(), t_w3_.data(), t_norm_.data(), up_w, up_s, block, B, dim,
+                                 ffn, stream_));                                                           // 1180-1183
+      const void* next_norm = l + 1 < n_layers ? model_->layers[l + 1].attn_norm.data() : model_->norm.data();
+      LCU_CHECK(lcu_batch_proj_norm(x, t_norm_.data(), t_silu_.data(), L.w2.data.data(), L.w2.scales.data(), block, B,
+                                    ffn, dim, next_norm, p.norm_eps, stream_));                            // 1185, 1129 / 1191
     }
-    // 1191-1209 for every row
-    LCU_CHECK(lcu_rmsnorm(t_norm_.data(), x, model_->norm.data(), B, dim, p.norm_eps, stream_));
+    // 1191-1209 for every row (the final norm is already in t_norm_)
     matmul(t_logits_.data(), t_norm_.data(), model_->output, B, 0.0f);
     LCU_CHECK(lcu_softmax_argmax_rows(t_probs_.data(), t_argmax_.data(), t_logits_.data(), B, vocab, temperature_,
                                       stream_));

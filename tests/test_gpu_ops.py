@@ -432,6 +432,88 @@ def test_attention_decode_twice_reuses_workspace(gpu):
     G.release()
 
 
+@pytest.mark.parametrize("B,dim,heads,ffn,u8", [(8, 4096, 32, 11008, False), (8, 4096, 32, 11008, True), (33, 1024, 8, 2816, False),
+                                                (3, 320, 2, 704, False), (1, 512, 4, 1408, True)])
+def test_batch_fused_steps_equal_their_separate_operators(gpu, B, dim, heads, ffn, u8):
+    """lcu_batch_qkv / lcu_batch_ffn_up / lcu_batch_proj_norm against the operators they fuse, bit for bit: on
+    shapes that take the split-K path (partial sums added up by the fused kernel), on shapes that do not
+    (dim 320: ragged K; one row) and with uint8 weights."""
+    G = gpu
+    L = G.L()
+    VP = G.B.vp
+    ctx, block = 16, (128 if u8 else 0)
+    table = VP()
+    G.B.check(L.lcu_rope_table_create(G.B.C.byref(table), ctx, dim // heads, 10000.0))
+    pos = np.arange(B, dtype=np.int32) % ctx
+    x = normal((B, dim), 0, 1700, 1.0)
+
+    def weights(rows, cols, stream):
+        w = normal((rows, cols), 0, stream, 0.02)
+        if not u8:
+            return G.dev_keep(w), None
+        c, sc = O.quantize_absmax_u8(w, 128)
+        return G.dev_keep(c), G.dev_keep(sc)
+
+    def arr(items):
+        return (VP * len(items))(*[(i.ptr if i is not None else None) for i in items])
+
+    def caches():
+        k = [G.dev_keep(np.zeros((ctx, dim), dtype=np.float16)) for _ in range(B)]
+        v = [G.dev_keep(np.zeros((ctx, dim), dtype=np.float16)) for _ in range(B)]
+        return k, v, G.dev_keep(np.array([d.ptr for d in k], dtype=np.uint64)), G.dev_keep(np.array([d.ptr for d in v], dtype=np.uint64))
+
+    xd, pd = G.dev_keep(x), G.dev_keep(pos)
+    # Wq, Wk, Wv + rotary + cache append
+    qkv = [weights(dim, dim, 1701 + g) for g in range(3)]
+    w_arr, s_arr = arr([w for w, _ in qkv]), arr([sc for _, sc in qkv])
+    res = []
+    for fused in (True, False):
+        kc, vc, kptr, vptr = caches()
+        q, kt, vt = G.empty((B, dim)), G.empty((B, dim)), G.empty((B, dim))
+        if fused:
+            G.B.check(L.lcu_batch_qkv(q.ptr, kt.ptr, vt.ptr, xd.ptr, w_arr, s_arr, block, B, dim, heads, kptr.ptr, vptr.ptr,
+                                      pd.ptr, table, ctx, None))
+        else:
+            outs = arr([q, kt, vt])
+            if u8:
+                G.B.check(L.lcu_gemm_f16u8_nt_multi(outs, xd.ptr, w_arr, s_arr, 3, B, dim, dim, block, 0.0, None))
+            else:
+                G.B.check(L.lcu_gemm_f16_nt_multi(outs, xd.ptr, w_arr, 3, B, dim, dim, 0.0, None))
+            G.B.check(L.lcu_rope_store_batch(q.ptr, kt.ptr, vt.ptr, kptr.ptr, vptr.ptr, pd.ptr, B, dim, heads, table, ctx, None))
+        res.append([G.host(q, (B, dim))] + [G.host(c, (ctx, dim)) for c in kc + vc])
+    for a, b in zip(*res):
+        assert (a.view(np.uint16) == b.view(np.uint16)).all()
+    assert np.abs(res[0][0].astype(np.float32)).max() > 0
+    # W1, W3 + SiLU
+    up = [weights(ffn, dim, 1710 + g) for g in range(2)]
+    w_arr, s_arr = arr([w for w, _ in up]), arr([sc for _, sc in up])
+    t1, t3, fused_out, sep_out = G.empty((B, ffn)), G.empty((B, ffn)), G.empty((B, ffn)), G.empty((B, ffn))
+    G.B.check(L.lcu_batch_ffn_up(fused_out.ptr, t1.ptr, t3.ptr, xd.ptr, w_arr, s_arr, block, B, dim, ffn, None))
+    outs = arr([t1, t3])
+    if u8:
+        G.B.check(L.lcu_gemm_f16u8_nt_multi(outs, xd.ptr, w_arr, s_arr, 2, B, dim, ffn, block, 0.0, None))
+    else:
+        G.B.check(L.lcu_gemm_f16_nt_multi(outs, xd.ptr, w_arr, 2, B, dim, ffn, 0.0, None))
+    G.B.check(L.lcu_silu_mul(sep_out.ptr, t1.ptr, t3.ptr, B * ffn, None))
+    assert (G.host(fused_out, (B, ffn)).view(np.uint16) == G.host(sep_out, (B, ffn)).view(np.uint16)).all()
+    # W2 with the residual + the next norm
+    h = normal((B, ffn), 0, 1720, 0.5)
+    hd = G.dev_keep(h)
+    w2, s2 = weights(dim, ffn, 1721)
+    nw = G.dev_keep(normal((dim,), 0, 1722, 1.0))
+    xa, xb, na, nb = G.dev(x), G.dev(x), G.empty((B, dim)), G.empty((B, dim))
+    G.B.check(L.lcu_batch_proj_norm(xa.ptr, na.ptr, hd.ptr, w2.ptr, s2.ptr if s2 else None, block, B, ffn, dim, nw.ptr, 1e-6, None))
+    if u8:
+        G.B.check(L.lcu_gemm_f16u8_nt(xb.ptr, hd.ptr, w2.ptr, s2.ptr, B, ffn, dim, block, 1.0, None))
+    else:
+        G.B.check(L.lcu_gemm_f16_nt(xb.ptr, hd.ptr, w2.ptr, B, ffn, dim, 1.0, None))
+    G.B.check(L.lcu_rmsnorm(nb.ptr, xb.ptr, nw.ptr, B, dim, 1e-6, None))
+    assert (G.host(xa, (B, dim)).view(np.uint16) == G.host(xb, (B, dim)).view(np.uint16)).all()
+    assert (G.host(na, (B, dim)).view(np.uint16) == G.host(nb, (B, dim)).view(np.uint16)).all()
+    G.release()
+    L.lcu_free(table)
+
+
 @pytest.mark.parametrize("n", [1, 5, 1000, 1024, 32000, 32003])
 def test_sample_row(gpu, n):
     # integer arithmetic on both sides: the drawn index must agree exactly

@@ -132,6 +132,42 @@ def test_decode_across_the_attention_form_boundary(gpu):
         o.close()
 
 
+MID = dict(dim=2048, multiple_of=256, n_heads=16, n_layers=2, n_vocab=1024)
+
+
+@pytest.mark.parametrize("q_type", [0, 1])
+def test_batched_decode_wide_model_vs_oracle(gpu, q_type):
+    """At this width the batched step's products take the split-K path and their partial sums are added up
+    by the fused kernels (rotary + cache append, SiLU, residual + next norm); five sequences, so the 32-row
+    tile is ragged; checked against the oracle's own contexts."""
+    G = gpu
+    om = O.Model(**MID, q_type=q_type, seed=31, weight_std=0.03)
+    gm = G.P.Model(**MID, q_type=q_type, seed=31, weight_std=0.03)
+    rng = np.random.default_rng(12)
+    prompts = [rng.integers(0, MID["n_vocab"], n).astype(np.int16) for n in (9, 2, 17, 1, 30)]
+    ocs = [O.Context(om, context_len=48, temperature=0.8) for _ in prompts]
+    bc = G.P.BatchContext(gm, len(prompts), context_len=48, temperature=0.8)
+    last = []
+    for b, pr in enumerate(prompts):
+        last.append(ocs[b].next_token(pr))
+        bc.next_token(b, pr)
+    for k in range(5):
+        want = [oc.next_token(np.array([t], dtype=np.int16), want=True) for oc, t in zip(ocs, last)]
+        got = bc.next_tokens(last)
+        logits, probs = bc.logits(), bc.probs()
+        for b, (otok, _, ologits, oprobs) in enumerate(want):
+            assert G.max_abs_rel(logits[b], ologits) <= TOL, (k, b)
+            assert G.max_abs_rel(probs[b], oprobs) <= 2 * TOL, (k, b)
+            lo = np.sort(ologits.astype(np.float32))
+            if lo[-1] - lo[-2] > 0.05:
+                assert got[b] == otok, (k, b)
+            last[b] = otok
+    T = [len(pr) + 5 for pr in prompts]
+    assert [bc.tokens_left(b) for b in range(len(prompts))] == [48 - t for t in T]
+    bc.close()
+    gm.close()
+
+
 @pytest.mark.parametrize("q_type", [0, 1])
 def test_batched_decode_vs_oracle(gpu, q_type):
     """llama_batch_context: three sequences with prompts of different lengths step together; every

@@ -240,6 +240,13 @@ def test_gemm_multi_matches_separate_calls(gpu, M, K, N, count):
             got = G.host(outs[g], (M, N))
             assert G.max_abs_rel(got, sep[g]) <= TOL and G.ulp_mismatch(got, sep[g]) < 0.05, g
             assert G.max_abs_rel(got, O.matmul_nt_u8(x, q[g][0], q[g][1], 128)) <= TOL, g
+    # beta = 1: every output starts from its own earlier contents
+    olds = [normal((M, N), 0, 1650 + g, 1.0) for g in range(count)]
+    for g in range(count):
+        G.B.check(L.lcu_h2d(outs[g].ptr, olds[g].ctypes.data_as(VP), olds[g].nbytes, None))
+    G.B.check(L.lcu_gemm_f16_nt_multi(out_arr, xd.ptr, w_arr, count, M, K, N, 1.0, None))
+    for g in range(count):
+        assert G.max_abs_rel(G.host(outs[g], (M, N)), O.matmul_nt(x, ws[g], beta=1.0, out=olds[g])) <= TOL, g
     assert L.lcu_gemm_f16_nt_multi(out_arr, xd.ptr, w_arr, 4, M, K, N, 0.0, None) == -2
     G.release()
 

@@ -114,6 +114,10 @@ int lcu_rope(void* out_dev, const void* in_dev, int rows, int cols, int n_heads,
              const void* table_dev, int table_positions, void* stream);
 /* softmax_rows, llama_cu.cu:433-499 (launch sites 1166, 1196); in place allowed */
 int lcu_softmax_rows(void* out_dev, const void* in_dev, int rows, int w, float temp, void* stream);
+/* e^x on n fp32 values with the exponential that every softmax and SiLU of this library takes
+ * (IEEE operations only, within one ulp; the reference calls CUDA's expf at llama_cu.cu:463, 497,
+ * 537).  Exported so that the host restatement of the same steps can be held to it bit for bit. */
+int lcu_exp_f32(void* out_dev, const void* in_dev, size_t n, void* stream);
 /* silu, llama_cu.cu:533-539 (launch site 1183) */
 int lcu_silu_mul(void* out_dev, const void* a_dev, const void* b_dev, size_t size, void* stream);
 /* embed / embed_uint8, llama_cu.cu:32-62 (launch sites 1090, 1094); ids are int16 */

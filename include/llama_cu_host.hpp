@@ -34,9 +34,9 @@ extern LLAMA_CU_API int matmul_type;
 // llama_cu.h:70-95 -- read-only file mapping, new read/write file of a given size, or anonymous memory
 struct LLAMA_CU_API mapped_buffer {
   mapped_buffer();
-  explicit mapped_buffer(std::string const& path);
+  mapped_buffer(std::string const& path);
   mapped_buffer(std::string const& path, size_t size);
-  explicit mapped_buffer(size_t size);
+  mapped_buffer(size_t size);
   ~mapped_buffer();
   mapped_buffer(mapped_buffer&& other);
   mapped_buffer& operator=(mapped_buffer&& other);
@@ -55,7 +55,7 @@ struct LLAMA_CU_API mapped_buffer {
 
 // llama_cu.h:97-107 -- selects a device for the lifetime of the object
 struct LLAMA_CU_API scoped_gpu {
-  explicit scoped_gpu(int device);
+  scoped_gpu(int device);
   ~scoped_gpu();
   scoped_gpu(scoped_gpu const&) = delete;
   scoped_gpu& operator=(scoped_gpu const&) = delete;
@@ -83,7 +83,7 @@ struct LLAMA_CU_API gpu_buffer_view {
 // llama_cu.h:124-134 -- owning device allocation
 struct LLAMA_CU_API gpu_buffer : public gpu_buffer_view {
   gpu_buffer() {}
-  explicit gpu_buffer(size_t size);
+  gpu_buffer(size_t size);
   gpu_buffer(gpu_buffer&& other);
   gpu_buffer& operator=(gpu_buffer&& other);
   ~gpu_buffer();
@@ -144,14 +144,14 @@ struct llama_token {
 };
 
 struct LLAMA_CU_API llama_vocabulary {
-  explicit llama_vocabulary(mapped_buffer const& buffer);
+  llama_vocabulary(mapped_buffer const& buffer);
   std::vector<short> tokenize(std::string_view text, bool bos);
   std::unordered_map<std::string, llama_token*> token_lookup;
   std::vector<llama_token> tokens;
 };
 
 struct LLAMA_CU_API llama_tokenizer {
-  explicit llama_tokenizer(llama_vocabulary const& vocab) : vocab_(vocab) {}
+  llama_tokenizer(llama_vocabulary const& vocab) : vocab_(vocab) {}
   void tokenize(std::string_view text, std::vector<short>& output);
 
  private:

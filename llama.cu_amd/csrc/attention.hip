@@ -111,7 +111,7 @@ __global__ __launch_bounds__(DEC_THREADS) void decode_attention_kernel(half_t* _
   __syncthreads();
   float s = 0.0f;
   if (tid < 256) {
-    for (int i = tid; i < T; i += 256) s += expf((float)sc[i] - m);
+    for (int i = tid; i < T; i += 256) s += exp_ieee((float)sc[i] - m);
   }
 #pragma unroll
   for (int off = 16; off > 0; off >>= 1) s += __shfl_xor(s, off, WAVE);
@@ -121,7 +121,7 @@ __global__ __launch_bounds__(DEC_THREADS) void decode_attention_kernel(half_t* _
 #pragma unroll
   for (int off = 4; off > 0; off >>= 1) total += __shfl_xor(total, off, WAVE);
   __syncthreads();
-  for (int i = tid; i < T; i += DEC_THREADS) sc[i] = round_f16(expf((float)sc[i] - m) / total);  // 497
+  for (int i = tid; i < T; i += DEC_THREADS) sc[i] = round_f16(exp_ieee((float)sc[i] - m) / total);  // 497
   __syncthreads();
 
   // ---- matmul_qkv, llama_cu.cu:511-531: group g adds rows g, g+64, ... in ascending order
@@ -230,9 +230,9 @@ __global__ __launch_bounds__(256) void dec_softmax_pv_kernel(half_t* __restrict_
   for (int i = tid; i < T; i += 256) m = fmaxf(m, (float)sc[i]);
   m = block256_max(m, red);
   float s = 0.0f;
-  for (int i = tid; i < T; i += 256) s += expf((float)sc[i] - m);
+  for (int i = tid; i < T; i += 256) s += exp_ieee((float)sc[i] - m);
   const float total = block256_sum_ref_order(s, red);
-  for (int i = tid; i < T; i += 256) sc[i] = round_f16(expf((float)sc[i] - m) / total);  // 497
+  for (int i = tid; i < T; i += 256) sc[i] = round_f16(exp_ieee((float)sc[i] - m) / total);  // 497
   __syncthreads();
   // matmul_qkv: row group g adds rows g, g+64, ... in ascending order, then the groups are added
   float acc[8];
@@ -420,11 +420,8 @@ __global__ __launch_bounds__(256) void prefill_attention_kernel(half_t* __restri
   prefetch_first(v);
   __syncthreads();
 
-  // ---- softmax over each row of the strip (llama_cu.cu:433-499): wave w owns rows w*8 .. w*8+7.
-  // exp is v_exp_f32 on x * log2(e) and the division a reciprocal multiply (both within an fp32
-  // ulp or two of the library calls, far below the fp16 rounding of the result): with the library
-  // expf the softmax was the longest phase of the kernel.
-  constexpr float LOG2E = 1.4426950408889634f;
+  // ---- softmax over each row of the strip (llama_cu.cu:433-499): wave w owns rows w*8 .. w*8+7;
+  // exp_ieee and a true division, as in every other softmax here
   for (int rr = 0; rr < BR / 4; ++rr) {
     // two neighbouring scores per lane and access (4 bytes: whole LDS words)
     half2_t* srow = reinterpret_cast<half2_t*>(Ss + (wave * (BR / 4) + rr) * SLD);
@@ -435,19 +432,17 @@ __global__ __launch_bounds__(256) void prefill_attention_kernel(half_t* __restri
       m = fmaxf(m, fmaxf((float)v.x, (float)v.y));
     }
     m = wave_max(m);
-    const float m2 = m * LOG2E;
     float s = 0.0f;
     for (int i = lane; i < pairs; i += WAVE) {
       const half2_t v = srow[i];
-      s += __builtin_amdgcn_exp2f(fmaf((float)v.x, LOG2E, -m2)) + __builtin_amdgcn_exp2f(fmaf((float)v.y, LOG2E, -m2));
+      s += exp_ieee((float)v.x - m) + exp_ieee((float)v.y - m);
     }
     s = wave_sum(s);
-    const float inv = __builtin_amdgcn_rcpf(s);
     for (int i = lane; i < pairs; i += WAVE) {
       const half2_t v = srow[i];
       half2_t p;
-      p.x = round_f16(__builtin_amdgcn_exp2f(fmaf((float)v.x, LOG2E, -m2)) * inv);
-      p.y = round_f16(__builtin_amdgcn_exp2f(fmaf((float)v.y, LOG2E, -m2)) * inv);
+      p.x = round_f16(exp_ieee((float)v.x - m) / s);
+      p.y = round_f16(exp_ieee((float)v.y - m) / s);
       srow[i] = p;
     }
   }

@@ -57,6 +57,34 @@ __device__ __forceinline__ half_t round_f16(float f) {
   return (half_t)f;
 }
 
+// e^x in fp32 from IEEE operations only (multiply, fused multiply-add, round to nearest even,
+// integer scaling), so that the host restatement of the same steps gives the same bits; within
+// one ulp of the true value, as the reference's expf is (llama_cu.cu:463, 497, 537 call CUDA's,
+// whose last bits no other platform reproduces either).  k = rne(x * log2 e); r = x - k * ln 2 with
+// ln 2 split in two; a degree-7 polynomial in r (Cephes' coefficients); the result scaled by 2^k in
+// two steps.  Results below the smallest normal number are returned as 0 and arguments above
+// 88.72283 as infinity, whatever the denormal mode of the machine.
+__device__ __forceinline__ float exp_ieee(float x) {
+  if (x > 88.72283f) return __builtin_inff();
+  if (x < -87.33654f) return 0.0f;
+  const float kf = __builtin_rintf(x * 1.44269504f);
+  float r = fmaf(kf, -0.693359375f, x);
+  r = fmaf(kf, 2.12194440e-4f, r);
+  float p = 1.9875691500e-4f;
+  p = fmaf(p, r, 1.3981999507e-3f);
+  p = fmaf(p, r, 8.3334519073e-3f);
+  p = fmaf(p, r, 4.1665795894e-2f);
+  p = fmaf(p, r, 1.6666665459e-1f);
+  p = fmaf(p, r, 5.0000001201e-1f);
+  p = fmaf(p * r, r, r) + 1.0f;
+  const int k = (int)kf;
+  const int k1 = k / 2, k2 = k - k1;
+  const float s1 = __builtin_bit_cast(float, (uint32_t)(k1 + 127) << 23);
+  const float s2 = __builtin_bit_cast(float, (uint32_t)(k2 + 127) << 23);
+  const float res = (p * s1) * s2;
+  return res < 1.17549435e-38f ? 0.0f : res;
+}
+
 // ---- wavefront reductions (all 64 lanes end with the result) ----
 template <int CTRL>
 __device__ __forceinline__ float dpp_f32(float v) {

@@ -89,11 +89,11 @@ __global__ __launch_bounds__(256) void softmax_rows_kernel(half_t* out, const ha
   m = block256_max(m, red);
   float s = 0.0f;
   for (int i = threadIdx.x; i < w; i += 256) {
-    s += expf((float)x[i] / temp - m);
+    s += exp_ieee((float)x[i] / temp - m);
   }
   const float total = block256_sum_ref_order(s, red);
   for (int i = threadIdx.x; i < w; i += 256) {
-    y[i] = round_f16(expf((float)x[i] / temp - m) / total);
+    y[i] = round_f16(exp_ieee((float)x[i] / temp - m) / total);
   }
 }
 
@@ -240,7 +240,7 @@ __global__ __launch_bounds__(1024) void softmax_argmax_kernel(half_t* __restrict
       if (tid + j * 1024 < n8) {
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
-          t[j][e] = expf(t[j][e] - m);
+          t[j][e] = exp_ieee(t[j][e] - m);
           s += t[j][e];
         }
       }
@@ -314,9 +314,9 @@ __global__ __launch_bounds__(1024) void softmax_argmax_kernel(half_t* __restrict
   for (int c = tid; c < n8; c += 1024) {
     const half8_t v = *reinterpret_cast<const half8_t*>(logits + (size_t)c * 8);
 #pragma unroll
-    for (int e = 0; e < 8; ++e) s += expf((float)v[e] / temp - m);
+    for (int e = 0; e < 8; ++e) s += exp_ieee((float)v[e] / temp - m);
   }
-  for (int i = n8 * 8 + tid; i < n; i += 1024) s += expf((float)logits[i] / temp - m);
+  for (int i = n8 * 8 + tid; i < n; i += 1024) s += exp_ieee((float)logits[i] / temp - m);
   s = wave_sum(s);
   if (lane == 0) sred[wave] = s;
   __syncthreads();
@@ -331,7 +331,7 @@ __global__ __launch_bounds__(1024) void softmax_argmax_kernel(half_t* __restrict
     half8_t p;
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
-      p[e] = round_f16(expf((float)v[e] / temp - m) / total);
+      p[e] = round_f16(exp_ieee((float)v[e] / temp - m) / total);
       const float f = (float)p[e];
       if (f > best) {  // ascending index within a thread: strict > keeps the first maximum
         best = f;
@@ -341,7 +341,7 @@ __global__ __launch_bounds__(1024) void softmax_argmax_kernel(half_t* __restrict
     *reinterpret_cast<half8_t*>(probs + (size_t)c * 8) = p;
   }
   for (int i = n8 * 8 + tid; i < n; i += 1024) {
-    const half_t p = round_f16(expf((float)logits[i] / temp - m) / total);
+    const half_t p = round_f16(exp_ieee((float)logits[i] / temp - m) / total);
     probs[i] = p;
     if ((float)p > best || ((float)p == best && i < idx)) {
       best = (float)p;
@@ -376,7 +376,7 @@ __global__ __launch_bounds__(1024) void softmax_argmax_kernel(half_t* __restrict
 // silu, llama_cu.cu:533-539
 __device__ __forceinline__ half_t silu_mul_one(half_t a, half_t b) {
   const float val = (float)a;
-  return round_f16(val / (1.0f + expf(-val)) * (float)b);
+  return round_f16(val / (1.0f + exp_ieee(-val)) * (float)b);
 }
 
 // eight elements per thread with 16-byte accesses (VEC: every pointer 16-byte aligned), the tail
@@ -429,6 +429,12 @@ __global__ void embed_u8_kernel(half_t* __restrict__ out, const short* __restric
     }
     out[(size_t)blockIdx.x * dim + i] = v;
   }
+}
+
+// exp_ieee on plain fp32 values (a check of the exponential every softmax and SiLU here uses)
+__global__ void exp_kernel(float* __restrict__ out, const float* __restrict__ in, size_t n) {
+  const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) out[i] = exp_ieee(in[i]);
 }
 
 // first maximum of n fp16 values compared as float, llama_cu.cu:1205-1209
@@ -776,6 +782,14 @@ int lcu_embed_u8(void* out_dev, const void* ids_dev, int n_ids, int dim, const v
   embed_u8_kernel<<<n_ids, 256, 0, as_stream(stream)>>>((half_t*)out_dev, (const short*)ids_dev, dim,
                                                         (const uint8_t*)codes_dev, (const half_t*)scales_dev, block,
                                                         n_vocab);
+  LCU_LAUNCH_CHECK();
+  return LCU_OK;
+}
+
+int lcu_exp_f32(void* out_dev, const void* in_dev, size_t n, void* stream) {
+  LCU_REQUIRE(out_dev && in_dev, "lcu_exp_f32: null pointer");
+  if (n == 0) return LCU_OK;
+  exp_kernel<<<(unsigned)((n + 255) / 256), 256, 0, as_stream(stream)>>>((float*)out_dev, (const float*)in_dev, n);
   LCU_LAUNCH_CHECK();
   return LCU_OK;
 }

@@ -945,8 +945,8 @@ __global__ __launch_bounds__(256) void reduce_silu_kernel(half_t* __restrict__ o
   const float2 g = sum_pair(part + (size_t)splits * mn, i, mn, splits);
   const float v0 = (float)round_f16(a.x), v1 = (float)round_f16(a.y);
   half2_t w;
-  w.x = round_f16(v0 / (1.0f + expf(-v0)) * (float)round_f16(g.x));
-  w.y = round_f16(v1 / (1.0f + expf(-v1)) * (float)round_f16(g.y));
+  w.x = round_f16(v0 / (1.0f + exp_ieee(-v0)) * (float)round_f16(g.x));
+  w.y = round_f16(v1 / (1.0f + exp_ieee(-v1)) * (float)round_f16(g.y));
   *reinterpret_cast<half2_t*>(out + i) = w;
 }
 

@@ -361,7 +361,7 @@ struct ffn_up_tasks {
   __device__ __forceinline__ void finish(int task, const float (&acc)[2]) const {
     const float val = (float)round_f16(acc[0]);
     const float gate = (float)round_f16(acc[1]);
-    out[task] = round_f16(val / (1.0f + expf(-val)) * gate);
+    out[task] = round_f16(val / (1.0f + exp_ieee(-val)) * gate);
   }
 };
 

@@ -53,6 +53,35 @@ inline float block_reduce_256(float* part, Op op) {
   return butterfly(warp, 8, op);
 }
 
+// e^x from IEEE operations only, step for step what exp_ieee in the HIP library does (its
+// csrc/common.hpp): k = rne(x * log2 e), r = x - k * ln 2 (ln 2 in two parts), Cephes' degree-7
+// polynomial, scaling by 2^k in two steps; below the smallest normal number 0, above 88.72283
+// infinity.  Within one ulp of e^x.  The reference calls CUDA's expf (llama_cu.cu:463, 497, 537),
+// whose last bits no host library reproduces; restating it with portable operations lets host and
+// GPU agree bit for bit wherever an exponential is taken.
+inline float exp_ieee(float x) {
+  if (x > 88.72283f) return INFINITY;
+  if (x < -87.33654f) return 0.0f;
+  const float kf = rintf(x * 1.44269504f);
+  float r = fmaf(kf, -0.693359375f, x);
+  r = fmaf(kf, 2.12194440e-4f, r);
+  float p = 1.9875691500e-4f;
+  p = fmaf(p, r, 1.3981999507e-3f);
+  p = fmaf(p, r, 8.3334519073e-3f);
+  p = fmaf(p, r, 4.1665795894e-2f);
+  p = fmaf(p, r, 1.6666665459e-1f);
+  p = fmaf(p, r, 5.0000001201e-1f);
+  p = fmaf(p * r, r, r) + 1.0f;
+  const int k = (int)kf;
+  const int k1 = k / 2, k2 = k - k1;
+  uint32_t b1 = (uint32_t)(k1 + 127) << 23, b2 = (uint32_t)(k2 + 127) << 23;
+  float s1, s2;
+  memcpy(&s1, &b1, 4);
+  memcpy(&s2, &b2, 4);
+  const float res = (p * s1) * s2;
+  return res < 1.17549435e-38f ? 0.0f : res;
+}
+
 inline float addf(float a, float b) { return a + b; }
 inline float maxf(float a, float b) { return fmaxf(a, b); }
 
@@ -117,6 +146,90 @@ inline void dot16x4(const float* x0, const float* x1, const float* x2, const flo
       acc[kk % 16] = fmaf(xs[i][kk], w[kk], acc[kk % 16]);
     }
     out[i] = butterfly(acc, 16, addf);
+  }
+}
+
+inline uint16_t epilogue(float acc, float beta, uint16_t old);
+
+// ---- flavour 2: the summation order of this repository's decode-time GEMV kernels (csrc/gemv.hip) ----
+// One 256-thread workgroup per output row(s): four wavefronts of 64 lanes.  K is cut into pieces
+// of `vec` elements (8 halves, or 16 uint8 codes); piece number c * 64 + lane of "chunk" c belongs
+// to lane `lane` of wavefront (c / U) % 4 (U = 2 for fp16 weights, 1 for uint8).  A lane keeps two
+// fp32 accumulators and walks its pieces in ascending order: fp16 weights alternate between the
+// accumulators element by element; uint8 weights go two by two (v_dot2_f32_f16), codes 0,1 of
+// every group of four to the first and codes 2,3 to the second.  The lane adds its two
+// accumulators, the 64 lanes are summed pairwise between neighbours (1, 2, 4, ... apart), and the
+// four wavefront sums are added in order.  All of it is fp32 fused multiply-add and add, so the
+// fp16 case is the kernel's result bit for bit; v_dot2_f32_f16 aligns and rounds its three
+// addends in a way of its own that is not restated here (restated as two fused multiply-adds), so
+// with uint8 weights this flavour follows the kernel to about one output in a hundred.
+inline float tree64(float* v) {
+  for (int s = 1; s < 64; s *= 2) {
+    for (int i = 0; i < 64; i += 2 * s) {
+      v[i] = v[i] + v[i + s];
+    }
+  }
+  return v[0];
+}
+
+inline float dot_gemv_order(const float* x, const float* w, int K, bool u8) {
+  const int vec = u8 ? 16 : 8, U = u8 ? 1 : 2, chunk = vec * 64;
+  float a0[4][64], a1[4][64];
+  for (int wv = 0; wv < 4; ++wv) {
+    for (int l = 0; l < 64; ++l) {
+      a0[wv][l] = 0.0f;
+      a1[wv][l] = 0.0f;
+    }
+  }
+  const int n_chunks = (K + chunk - 1) / chunk;
+  for (int c = 0; c < n_chunks; ++c) {
+    const int wv = (c / U) % 4;
+    for (int l = 0; l < 64; ++l) {
+      const int kk = c * chunk + l * vec;
+      if (kk >= K) break;
+      float p0 = a0[wv][l], p1 = a1[wv][l];
+      if (u8) {
+        for (int j = 0; j < 16; j += 4) {
+          p0 = fmaf(w[kk + j + 1], x[kk + j + 1], fmaf(w[kk + j], x[kk + j], p0));
+          p1 = fmaf(w[kk + j + 3], x[kk + j + 3], fmaf(w[kk + j + 2], x[kk + j + 2], p1));
+        }
+      } else {
+        for (int e = 0; e < 8; e += 2) {
+          p0 = fmaf(w[kk + e], x[kk + e], p0);
+          p1 = fmaf(w[kk + e + 1], x[kk + e + 1], p1);
+        }
+      }
+      a0[wv][l] = p0;
+      a1[wv][l] = p1;
+    }
+  }
+  float acc = 0.0f;
+  for (int wv = 0; wv < 4; ++wv) {
+    float lanes[64];
+    for (int l = 0; l < 64; ++l) {
+      lanes[l] = a0[wv][l] + a1[wv][l];
+    }
+    acc += tree64(lanes);
+  }
+  return acc;
+}
+
+void matvec_gemv_order(uint16_t* out, const uint16_t* lhs, const uint16_t* rhs_h, const uint8_t* rhs_q,
+                       const uint16_t* scales, int K, int N, int block, float beta) {
+  std::vector<float> xf(K);
+  row_to_float(xf.data(), lhs, K);
+#pragma omp parallel
+  {
+    std::vector<float> wf(K);
+#pragma omp for schedule(static)
+    for (int n = 0; n < N; ++n) {
+      if (rhs_q) {
+        row_u8_to_float(wf.data(), rhs_q + (size_t)n * K, scales + (size_t)n * (K / block), K, block);
+      } else {
+        row_to_float(wf.data(), rhs_h + (size_t)n * K, K);
+      }
+      out[n] = epilogue(dot_gemv_order(xf.data(), wf.data(), K, rhs_q != nullptr), beta, out[n]);
+    }
   }
 }
 
@@ -239,6 +352,10 @@ void orc_matmul_nt(uint16_t* out, const uint16_t* lhs, const uint16_t* rhs, int 
     }
     return;
   }
+  if (flavour == 2 && M == 1 && K % 8 == 0) {
+    matvec_gemv_order(out, lhs, rhs, nullptr, nullptr, K, N, 1, beta);
+    return;
+  }
   matmul_tiled(out, lhs, rhs, nullptr, nullptr, M, K, N, 1, beta);
 }
 
@@ -263,6 +380,10 @@ void orc_matmul_nt_u8(uint16_t* out, const uint16_t* lhs, const uint8_t* codes,
         out[o] = epilogue(sum, beta, out[o]);
       }
     }
+    return;
+  }
+  if (flavour == 2 && M == 1 && K % 16 == 0) {
+    matvec_gemv_order(out, lhs, nullptr, codes, scales, K, N, block, beta);
     return;
   }
   matmul_tiled(out, lhs, nullptr, codes, scales, M, K, N, block, beta);
@@ -363,13 +484,13 @@ void orc_softmax_rows(uint16_t* out, const uint16_t* in, int rows, int w, float 
     for (int t = 0; t < 256; ++t) {
       float s = 0.0f;
       for (int i = t; i < w; i += 256) {
-        s += expf(h2f(x[i]) / temp - max_val);
+        s += exp_ieee(h2f(x[i]) / temp - max_val);
       }
       part[t] = s;
     }
     const float sum_exp = block_reduce_256(part, addf);
     for (int i = 0; i < w; ++i) {
-      y[i] = f2h(expf(h2f(x[i]) / temp - max_val) / sum_exp);
+      y[i] = f2h(exp_ieee(h2f(x[i]) / temp - max_val) / sum_exp);
     }
   }
 }
@@ -403,7 +524,7 @@ void orc_silu_mul(uint16_t* out, const uint16_t* a, const uint16_t* b, size_t si
 #pragma omp parallel for schedule(static)
   for (size_t i = 0; i < size; ++i) {
     float val = h2f(a[i]);
-    out[i] = f2h(val / (1.0f + expf(-val)) * h2f(b[i]));
+    out[i] = f2h(val / (1.0f + exp_ieee(-val)) * h2f(b[i]));
   }
 }
 
@@ -664,6 +785,96 @@ void orc_context_kv(orc_context* c, int layer, uint16_t* k_rot, uint16_t* v, int
   if (v) memcpy(v, c->v[layer].data(), n * 2);
 }
 
+// ---- flavour 2, one new token: attention and the logits softmax in the order of the HIP kernels ----
+// csrc/attention.hip, decode: a cached row's 128-wide dot product is taken by 16 lanes, 8 elements
+// each in ascending order (fused multiply-adds from 0), the 16 lane sums added pairwise between
+// neighbours; the softmax is softmax_rows as above; the weighted sum of V is taken by 64 row groups,
+// group g adding rows g, g + 64, ... in ascending order, and the 64 group sums are added in order
+// from 0.  head_dim must be 128.
+static void attention_decode_kernel_order(uint16_t* out, const uint16_t* q, const uint16_t* k, const uint16_t* v,
+                                          int T, int dim, int n_heads) {
+  const float denom = sqrtf(128.0f);
+#pragma omp parallel for schedule(static)
+  for (int h = 0; h < n_heads; ++h) {
+    std::vector<uint16_t> sc(T);
+    for (int p = 0; p < T; ++p) {
+      float lane[16];
+      for (int sub = 0; sub < 16; ++sub) {
+        float s = 0.0f;
+        for (int e = 0; e < 8; ++e) {
+          const int col = h * 128 + sub * 8 + e;
+          s = fmaf(h2f(q[col]), h2f(k[(size_t)p * dim + col]), s);
+        }
+        lane[sub] = s;
+      }
+      for (int st = 1; st < 16; st *= 2) {
+        for (int i = 0; i < 16; i += 2 * st) lane[i] = lane[i] + lane[i + st];
+      }
+      sc[p] = f2h(lane[0] / denom);
+    }
+    // softmax_rows, temp 1 (llama_cu.cu:433-499)
+    float part[256];
+    for (int t = 0; t < 256; ++t) {
+      float m = -INFINITY;
+      for (int i = t; i < T; i += 256) m = fmaxf(m, h2f(sc[i]));
+      part[t] = m;
+    }
+    const float max_val = block_reduce_256(part, maxf);
+    for (int t = 0; t < 256; ++t) {
+      float s = 0.0f;
+      for (int i = t; i < T; i += 256) s += exp_ieee(h2f(sc[i]) - max_val);
+      part[t] = s;
+    }
+    const float sum_exp = block_reduce_256(part, addf);
+    for (int i = 0; i < T; ++i) sc[i] = f2h(exp_ieee(h2f(sc[i]) - max_val) / sum_exp);
+    for (int j = 0; j < 128; ++j) {
+      const int col = h * 128 + j;
+      float o = 0.0f;
+      for (int g = 0; g < 64; ++g) {
+        float acc = 0.0f;
+        for (int p = g; p < T; p += 64) acc = fmaf(h2f(sc[p]), h2f(v[(size_t)p * dim + col]), acc);
+        o += acc;
+      }
+      out[col] = f2h(o);
+    }
+  }
+}
+
+// softmax_argmax_kernel of csrc/elementwise.hip (n a multiple of 8, at most 32768): thread t of 1024
+// owns the 8-element pieces t, t + 1024, ... and adds their exponentials in ascending order; the 64
+// lanes of a wavefront are summed pairwise between neighbours; the 16 wavefront sums are added in
+// order from 0.  Everything else is softmax_rows.
+static void softmax_logits_kernel_order(uint16_t* y, const uint16_t* x, int n, float temp) {
+  float m = -INFINITY;
+  for (int i = 0; i < n; ++i) m = fmaxf(m, h2f(x[i]) / temp);
+  float total = 0.0f;
+  for (int wv = 0; wv < 16; ++wv) {
+    float lanes[64];
+    for (int l = 0; l < 64; ++l) {
+      float s = 0.0f;
+      for (int c = wv * 64 + l; c < n / 8; c += 1024) {
+        for (int e = 0; e < 8; ++e) s += exp_ieee(h2f(x[c * 8 + e]) / temp - m);
+      }
+      lanes[l] = s;
+    }
+    total += tree64(lanes);
+  }
+  for (int i = 0; i < n; ++i) y[i] = f2h(exp_ieee(h2f(x[i]) / temp - m) / total);
+}
+
+void orc_exp_f32(float* out, const float* in, size_t n) {
+  for (size_t i = 0; i < n; ++i) out[i] = exp_ieee(in[i]);
+}
+
+void orc_attention_decode_kernel_order(uint16_t* out, const uint16_t* q, const uint16_t* k, const uint16_t* v, int T,
+                                       int dim, int n_heads) {
+  attention_decode_kernel_order(out, q, k, v, T, dim, n_heads);
+}
+
+void orc_softmax_logits_kernel_order(uint16_t* out, const uint16_t* in, int n, float temp) {
+  softmax_logits_kernel_order(out, in, n, temp);
+}
+
 int orc_context_next_token(orc_context* c, const int16_t* tokens, int n, uint16_t* hidden,
                            uint16_t* logits_out, uint16_t* probs_out) {
   orc_model* m = c->model;
@@ -696,9 +907,13 @@ int orc_context_next_token(orc_context* c, const int16_t* tokens, int n, uint16_
       krot = kc;
     }
     mm(c, vc + (size_t)sp * dim, norm.data(), L.wv, n, 0.0f);                      // 1156
-    orc_matmul_qk(qk.data(), xq.data(), krot, n, T, dim, H, sp);                   // 1163
-    orc_softmax_rows(qk.data(), qk.data(), H * n, T, 1.0f);                        // 1166
-    orc_matmul_qkv(att.data(), qk.data(), vc, n, T, dim, H);                       // 1170
+    if (c->flavour == 2 && n == 1 && dim == H * 128) {
+      attention_decode_kernel_order(att.data(), xq.data(), krot, vc, T, dim, H);   // 1163-1170
+    } else {
+      orc_matmul_qk(qk.data(), xq.data(), krot, n, T, dim, H, sp);                 // 1163
+      orc_softmax_rows(qk.data(), qk.data(), H * n, T, 1.0f);                      // 1166
+      orc_matmul_qkv(att.data(), qk.data(), vc, n, T, dim, H);                     // 1170
+    }
     mm(c, x.data(), att.data(), L.wo, n, 1.0f);                                    // 1174
     orc_rms_norm(norm.data(), x.data(), L.ffn_norm.data(), n, dim, m->norm_eps);   // 1176
     mm(c, w1.data(), norm.data(), L.w1, n, 0.0f);                                  // 1180
@@ -711,7 +926,12 @@ int orc_context_next_token(orc_context* c, const int16_t* tokens, int n, uint16_
   std::vector<uint16_t> logits(m->n_vocab);
   mm(c, logits.data(), norm.data() + (size_t)(n - 1) * dim, m->output, 1, 0.0f);   // 1194-1195
   if (logits_out) memcpy(logits_out, logits.data(), logits.size() * 2);
-  orc_softmax_rows(logits.data(), logits.data(), 1, m->n_vocab, c->temperature);   // 1196
+  if (c->flavour == 2 && m->n_vocab % 8 == 0 && m->n_vocab <= 32768) {
+    std::vector<uint16_t> raw(logits);
+    softmax_logits_kernel_order(logits.data(), raw.data(), m->n_vocab, c->temperature);
+  } else {
+    orc_softmax_rows(logits.data(), logits.data(), 1, m->n_vocab, c->temperature);  // 1196
+  }
   if (probs_out) memcpy(probs_out, logits.data(), logits.size() * 2);
   c->start_pos += n;                                                               // 1201
   return orc_argmax_first(logits.data(), m->n_vocab);                              // 1205-1209

@@ -12,6 +12,9 @@
  *       hand-computed known-answer block, the exhaustive 65536-input sweep against numpy
  *       float32/float16 and the absmax/code-range invariants (tests/test_oracle_quant.py).
  *   orc_matmul_nt[_u8] : pinned by float64 brute force, identity / one-hot / beta special cases.
+ *   exponentials (softmax, SiLU): the reference calls CUDA's expf, whose last bits no host library
+ *       reproduces; restated with IEEE operations only (exp_ieee, within one ulp, pinned against
+ *       float64 exp in tests/test_oracle_ops.py) so that host and GPU agree bit for bit.
  *   orc_rms_norm, orc_rotary, orc_softmax_rows, orc_silu_mul, orc_matmul_qk, orc_matmul_qkv,
  *   orc_embed[_u8], orc_argmax_first : pinned by closed forms and float64 restatements written
  *       independently in numpy (tests/test_oracle_ops.py).
@@ -48,7 +51,16 @@ void orc_dequantize_absmax_u8(uint16_t* out, const uint16_t* scales, const uint8
  * flavour 1: the tensor-core kernels llama_cu.cu:150-220, 225-285, 294-366: fp16 operands
  *            (u8 weights first rounded to fp16 by dequantize_absmax_one, 287-289), fp32
  *            accumulation in an order the hardware fixes; restated with 16 interleaved partial
- *            sums and a pairwise tree. */
+ *            sums and a pairwise tree.
+ * flavour 2: as flavour 1, except that a single row (M == 1) is summed in the order of this
+ *            repository's own decode GEMV kernels (lane-strided partial sums, a pairwise tree over
+ *            the 64 lanes, the four wavefronts in order; see dot_gemv_order in oracle.cpp), and a
+ *            context created with it also takes the attention and the logits softmax of a
+ *            one-token call in the order of the HIP kernels.  Any fp32 order is as good a restatement
+ *            of the reference's tensor-core sums as another (their order is the hardware's); this
+ *            one lets a decode step be compared with the GPU bit for bit (fp16 weights) instead
+ *            of within a tolerance.  Pinned by the same float64 / identity / one-hot checks as the
+ *            other flavours (tests/test_oracle_ops.py). */
 void orc_matmul_nt(uint16_t* out, const uint16_t* lhs, const uint16_t* rhs, int M, int K, int N,
                    float beta, int flavour);
 void orc_matmul_nt_u8(uint16_t* out, const uint16_t* lhs, const uint8_t* codes,
@@ -96,6 +108,18 @@ uint64_t orc_step_random(uint64_t seed, uint64_t step);
  * so its own result is only defined to fp32 summation accuracy).  Pinned by closed forms:
  * identical arrays -> 0, a constant offset -> {c^2, c, c}, one differing element. */
 void orc_error_stats(float* out3, const uint16_t* a, const uint16_t* b, size_t n);
+
+/* e^x as every softmax and SiLU of this oracle takes it: IEEE operations only (the reference calls
+ * CUDA's expf, llama_cu.cu:463, 497, 537); pinned against float64 exp to one ulp. */
+void orc_exp_f32(float* out, const float* in, size_t n);
+/* Attention of one new token (q [dim], the first T rows of k (rotated) and v [T][dim], head_dim 128)
+ * and softmax with temperature over one row of n logits (n a multiple of 8 up to 32768): the
+ * arithmetic of llama_cu.cu:400-428, 433-499, 511-531 with the sums taken in the order of this
+ * repository's HIP kernels (what a context of matmul flavour 2 uses for one-token calls).  Pinned
+ * against orc_matmul_qk / orc_softmax_rows / orc_matmul_qkv within fp32 summation accuracy. */
+void orc_attention_decode_kernel_order(uint16_t* out, const uint16_t* q, const uint16_t* k, const uint16_t* v, int T,
+                                       int dim, int n_heads);
+void orc_softmax_logits_kernel_order(uint16_t* out, const uint16_t* in, int n, float temp);
 
 /* ---- whole model: llama_cu.cu:882-1210 with seeded random weights instead of files ---- */
 typedef struct orc_model orc_model;

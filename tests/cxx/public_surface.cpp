@@ -60,6 +60,17 @@ int main(int argc, char**) {
   ok = ok && t.id == 0 && t.score <= 0.0f && !t.text.empty() && vocab.token_lookup.count(t.text) == 1;
   llama_tokenizer tokenizer(vocab);
   tokenizer.tokenize(std::string_view("hello"), ids);
+  // the reference's single-argument constructors are not explicit (llama_cu.h:72-74, 98, 126, 323,
+  // 330): each type converts implicitly from its argument
+  mapped_buffer by_path = std::string("models/7B/params");
+  mapped_buffer by_size = (size_t)4096;
+  gpu_buffer by_bytes = (size_t)256;
+  auto takes_scope = [](scoped_gpu const&) {};
+  takes_scope(0);
+  llama_vocabulary by_buffer = vocab_file;
+  llama_tokenizer by_vocab = vocab;
+  by_vocab.tokenize(std::string_view("hello"), ids);
+  ok = ok && by_path.is_ok() && by_size.is_ok() && by_bytes.is_ok() && !by_buffer.tokens.empty();
   std::unique_ptr<llama_model> model = llama_model::load(p, part, std::string("models/7B"));
   ok = ok && model && model->params.dim == p.dim && model->partition.output_gpu == part.output_gpu;
   std::unique_ptr<llama_context> context = llama_context::create(model.get());

@@ -4,7 +4,9 @@
     python tests/golden/make_greedy_fixture.py llama30b_u8 [seed]
 
 Each fixture holds the model shape, the seeds, the 512 prompt token ids, the 128 greedy tokens the
-oracle produces (tensor-core flavour of the matmul, temperature 0.8 as main.cpp:58), and for every
+oracle produces (matmul flavour 2: the 512-token prompt goes through the tensor-core-like flavour,
+every one-token step through the summation order of the HIP decode kernels, so that a decode step
+can be held to the GPU bit for bit; temperature 0.8 as main.cpp:58), and for every
 step the two largest fp16 logits with their token ids and the two largest probabilities, so that
 a mismatch in a GPU run can be attributed to a near-tie.  Only the oracle runs here; nothing from the reference is
 imported or executed.
@@ -37,7 +39,7 @@ def main():
     t0 = time.time()
     model = O.Model(norm_eps=1e-6, qblock=128, seed=seed, weight_std=0.02, **cfg)
     print("model built in %.1fs (ffn %d)" % (time.time() - t0, model.ffn), flush=True)
-    ctx = O.Context(model, context_len=2048, temperature=0.8, flavour=1)
+    ctx = O.Context(model, context_len=2048, temperature=0.8, flavour=2)
     prompt = np.random.default_rng(seed).integers(0, cfg["n_vocab"], prompt_len).astype(np.int16)
     tokens, top, top_ids = [], [], []
     feed = prompt
@@ -53,7 +55,7 @@ def main():
         top_ids.append([int(order[0]), int(order[1])])
         feed = np.array([tok], dtype=np.int16)
         print("step %d token %d logit margin %.5f (%.1fs)" % (step, tok, lo[1] - lo[0], time.time() - t1), flush=True)
-    out = dict(name=name, seed=seed, weight_std=0.02, norm_eps=1e-6, qblock=128, temperature=0.8, context_len=2048,
+    out = dict(name=name, matmul_flavour=2, seed=seed, weight_std=0.02, norm_eps=1e-6, qblock=128, temperature=0.8, context_len=2048,
                prompt=[int(t) for t in prompt], tokens=tokens, top2_logits_probs=top, top2_ids=top_ids, **cfg)
     path = os.path.join(HERE, "%s_seed%d_greedy.json" % (name, seed))
     with open(path, "w") as f:

@@ -39,6 +39,12 @@ def lib():
         L.orc_softmax_rows.argtypes = [vp, vp, i, i, f]
         L.orc_matmul_qkv.argtypes = [vp, vp, vp, i, i, i, i]
         L.orc_silu_mul.argtypes = [vp, vp, vp, sz]
+        L.orc_exp_f32.argtypes = [vp, vp, sz]
+        L.orc_exp_f32.restype = None
+        L.orc_attention_decode_kernel_order.argtypes = [vp, vp, vp, vp, i, i, i]
+        L.orc_attention_decode_kernel_order.restype = None
+        L.orc_softmax_logits_kernel_order.argtypes = [vp, vp, i, f]
+        L.orc_softmax_logits_kernel_order.restype = None
         L.orc_embed.argtypes = [vp, vp, i, i, vp]
         L.orc_embed_u8.argtypes = [vp, vp, i, i, vp, vp, i]
         L.orc_error_stats.argtypes = [vp, vp, vp, sz]
@@ -170,6 +176,29 @@ def matmul_qkv(p, v, n_heads):
 def attention(q, k, v, n_heads, start_pos):
     """matmul_qk -> softmax_rows -> matmul_qkv, llama_cu.cu:1161-1171."""
     return matmul_qkv(softmax_rows(matmul_qk(q, k, n_heads, start_pos)), v, n_heads)
+
+
+def exp_f32(x):
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    out = np.empty_like(x)
+    lib().orc_exp_f32(_p(out), _p(x), x.size)
+    return out
+
+
+def attention_decode_kernel_order(q, k, v, n_heads):
+    """one new token against T cached rows, sums in the order of the HIP kernels"""
+    q, k, v = _f16(q), _f16(k), _f16(v)
+    T, dim = k.shape
+    out = np.empty((1, dim), dtype=np.float16)
+    lib().orc_attention_decode_kernel_order(_p(out), _p(q), _p(k), _p(v), T, dim, n_heads)
+    return out
+
+
+def softmax_logits_kernel_order(x, temp):
+    x = _f16(x)
+    out = np.empty_like(x)
+    lib().orc_softmax_logits_kernel_order(_p(out), _p(x), x.size, temp)
+    return out
 
 
 def silu_mul(a, b):

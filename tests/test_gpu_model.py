@@ -306,6 +306,30 @@ def test_sampling_follows_the_step_random_sequence(gpu):
         o.close()
 
 
+@pytest.mark.parametrize("cfg,steps", [(dict(dim=512, multiple_of=128, n_heads=4, n_layers=3, n_vocab=2048), 40),
+                                        (dict(dim=4096, multiple_of=256, n_heads=32, n_layers=2, n_vocab=32000), 12)])
+def test_decode_steps_bit_exact_against_kernel_order_oracle(gpu, cfg, steps):
+    """Tokens fed one at a time (every call is a decode step): with fp16 weights the oracle's flavour 2
+    restates the summation order of every kernel on that path, and the exponential and the RoPE table
+    are shared arithmetic, so hidden state, logits, probabilities and token agree on every bit."""
+    G = gpu
+    om = O.Model(**cfg, seed=3, weight_std=0.05)
+    gm = G.P.Model(**cfg, seed=3, weight_std=0.05)
+    oc = O.Context(om, context_len=64, temperature=0.8, flavour=2)
+    gc = G.P.Context(gm, context_len=64, temperature=0.8)
+    tok = 7
+    for step in range(steps):
+        otok, ohid, ologits, oprobs = oc.next_token([tok], want=True)
+        gtok = gc.next_token([tok])
+        assert G.ulp_mismatch(gc.hidden(1), ohid) == 0.0, step
+        assert G.ulp_mismatch(gc.logits(), ologits) == 0.0, step
+        assert G.ulp_mismatch(gc.probs(), oprobs) == 0.0, step
+        assert gtok == otok, step
+        tok = otok
+    gc.close()
+    gm.close()
+
+
 def test_one_llama7b_layer_prefill_512_then_decode_at_2048(gpu):
     """One LLaMA-7B decoder layer: 512-token prefill, chunked prefill up to 2047 cached tokens,
     then a single-token decode at KV length 2048."""

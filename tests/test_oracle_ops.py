@@ -21,7 +21,7 @@ def f16(a):
 
 
 # ------------------------------------------------------------------ matmul
-@pytest.mark.parametrize("flavour", [0, 1])
+@pytest.mark.parametrize("flavour", [0, 1, 2])
 @pytest.mark.parametrize("M,K,N", [(1, 256, 64), (5, 272, 33), (16, 1024, 128), (3, 40, 7)])
 def test_matmul_vs_float64(flavour, M, K, N):
     x = f16(RNG.normal(0, 1, (M, K)))
@@ -32,7 +32,7 @@ def test_matmul_vs_float64(flavour, M, K, N):
     assert np.max(np.abs(out.astype(np.float64) - ref)) <= np.max(np.abs(ref)) * 2.0 ** -10
 
 
-@pytest.mark.parametrize("flavour", [0, 1])
+@pytest.mark.parametrize("flavour", [0, 1, 2])
 def test_matmul_exact_cases(flavour):
     K = 128
     x = f16(RNG.normal(0, 1, (4, K)))
@@ -51,7 +51,7 @@ def test_matmul_exact_cases(flavour):
     assert out[1, 2] == 6 and np.count_nonzero(out) == 1
 
 
-@pytest.mark.parametrize("flavour", [0, 1])
+@pytest.mark.parametrize("flavour", [0, 1, 2])
 def test_matmul_beta_residual(flavour):
     x = f16(RNG.normal(0, 1, (3, 256)))
     w = f16(RNG.normal(0, 0.02, (20, 256)))
@@ -64,7 +64,7 @@ def test_matmul_beta_residual(flavour):
     assert np.isfinite(O.matmul_nt(x, w, beta=0.0, out=junk, flavour=flavour)).all()
 
 
-@pytest.mark.parametrize("flavour", [0, 1])
+@pytest.mark.parametrize("flavour", [0, 1, 2])
 def test_matmul_u8_vs_float64_and_dequant_route(flavour):
     K, N, M, block = 512, 40, 3, 128
     w = f16(RNG.normal(0, 0.02, (N, K)))
@@ -86,6 +86,121 @@ def test_matmul_row_independence():
     full = O.matmul_nt(x, w)
     for r in (0, 4, 8):
         assert (O.matmul_nt(x[r:r + 1], w).view(np.uint16) == full[r:r + 1].view(np.uint16)).all()
+
+
+# ------------------------------------------------------------------ flavour 2 (one row in the order of the HIP GEMV kernels)
+def gemv_order_numpy(x, w, u8):
+    """Independent restatement of dot_gemv_order: products of two halves are exact in fp32, so every
+    fused multiply-add is a plain fp32 addition of an exact product."""
+    K = x.size
+    vec, U = (16, 1) if u8 else (8, 2)
+    chunk = vec * 64
+    acc = np.zeros((4, 64, 2), dtype=np.float32)
+    prod = (x.astype(np.float32) * w.astype(np.float32)).astype(np.float32)
+    lanes = np.arange(64)
+    for c in range((K + chunk - 1) // chunk):
+        wave = (c // U) % 4
+        kk = c * chunk + lanes * vec
+        ok = kk < K
+        for e in range(vec):
+            which = (e % 4) // 2 if u8 else e % 2
+            idx = np.where(ok, kk + e, 0)
+            acc[wave, :, which] = np.where(ok, (acc[wave, :, which] + prod[idx]).astype(np.float32), acc[wave, :, which])
+    total = np.float32(0)
+    for wave in range(4):
+        v = (acc[wave, :, 0] + acc[wave, :, 1]).astype(np.float32)
+        step = 1
+        while step < 64:
+            v[::2 * step] = (v[::2 * step] + v[step::2 * step]).astype(np.float32)
+            step *= 2
+        total = np.float32(total + v[0])
+    return total
+
+
+@pytest.mark.parametrize("K", [8, 512, 1032, 4096, 11008])
+def test_single_row_kernel_order_fp16(K):
+    x = f16(RNG.normal(0, 1, (1, K)))
+    w = f16(RNG.normal(0, 0.02, (5, K)))
+    out = O.matmul_nt(x, w, flavour=2)
+    ref64 = x.astype(np.float64) @ w.astype(np.float64).T
+    assert np.max(np.abs(out.astype(np.float64) - ref64)) <= np.max(np.abs(ref64)) * 2.0 ** -10
+    want = np.array([[gemv_order_numpy(x[0], w[n], False) for n in range(5)]], dtype=np.float32).astype(np.float16)
+    assert (out.view(np.uint16) == want.view(np.uint16)).all()
+    # residual: one rounding of the fp32 sum
+    old = f16(RNG.normal(0, 1, (1, 5)))
+    out = O.matmul_nt(x, w, beta=1.0, out=old, flavour=2)
+    want = np.array([[np.float32(gemv_order_numpy(x[0], w[n], False) + np.float32(old[0, n])) for n in range(5)]],
+                    dtype=np.float32).astype(np.float16)
+    assert (out.view(np.uint16) == want.view(np.uint16)).all()
+    # exact cases: a one-hot row picks a column of w
+    onehot = np.zeros((1, K), dtype=np.float16)
+    onehot[0, K // 3] = 1
+    assert (O.matmul_nt(onehot, w, flavour=2)[0].view(np.uint16) == w[:, K // 3].view(np.uint16)).all()
+
+
+@pytest.mark.parametrize("K", [128, 1024, 6656])
+def test_single_row_kernel_order_u8(K):
+    block = 128
+    w = f16(RNG.normal(0, 0.02, (4, K)))
+    x = f16(RNG.normal(0, 1, (1, K)))
+    codes, scales = O.quantize_absmax_u8(w, block)
+    wd = O.dequantize_absmax_u8(codes, scales, block)
+    out = O.matmul_nt_u8(x, codes, scales, block, flavour=2)
+    want = np.array([[gemv_order_numpy(x[0], wd[n], True) for n in range(4)]], dtype=np.float32).astype(np.float16)
+    assert (out.view(np.uint16) == want.view(np.uint16)).all()
+    ref64 = x.astype(np.float64) @ wd.astype(np.float64).T
+    assert np.max(np.abs(out.astype(np.float64) - ref64)) <= np.max(np.abs(ref64)) * 2.0 ** -10
+
+
+def test_exp_ieee_against_float64():
+    x = np.concatenate([np.linspace(-90, 89, 200001), RNG.normal(0, 3, 100000), RNG.uniform(-20, 0, 100000),
+                        [0.0, -0.0, 1.0, -1.0, 88.7, -87.3]]).astype(np.float32)
+    got = O.exp_f32(x)
+    ref = np.exp(x.astype(np.float64))
+    normal = (ref >= 1.18e-38) & (ref < 3.4e38)
+    ulp = np.spacing(ref[normal].astype(np.float32)).astype(np.float64)
+    assert np.max(np.abs(got[normal].astype(np.float64) - ref[normal]) / ulp) <= 1.05  # CUDA documents 2 ulp for expf
+    assert got[x == 0].tolist() == [1.0] * int((x == 0).sum())
+    special = O.exp_f32(np.array([-np.inf, -200.0, 89.0, np.inf, np.nan], dtype=np.float32))
+    assert special[0] == 0 and special[1] == 0 and np.isposinf(special[2]) and np.isposinf(special[3]) and np.isnan(special[4])
+    # monotone on a dense grid (a softmax must not reorder its inputs)
+    grid = np.linspace(-30, 10, 400001).astype(np.float32)
+    assert (np.diff(O.exp_f32(grid)) >= 0).all()
+
+
+@pytest.mark.parametrize("T", [1, 7, 64, 577, 1500])
+def test_attention_decode_kernel_order(T):
+    n_heads, dim = 3, 384
+    q = f16(RNG.normal(0, 1, (1, dim)))
+    k = f16(RNG.normal(0, 1, (T, dim)))
+    v = f16(RNG.normal(0, 1, (T, dim)))
+    got = O.attention_decode_kernel_order(q, k, v, n_heads)
+    # same arithmetic as the reference-ordered chain: scores may differ by the last fp16 bit, so the
+    # output follows it to fp16 rounding accuracy, and float64 attention within the usual bound
+    ref = O.attention(q, k, v, n_heads, T - 1)
+    assert np.max(np.abs(got.astype(np.float64) - ref.astype(np.float64))) <= 2.0 ** -8 * np.max(np.abs(ref.astype(np.float64)))
+    q64, k64, v64 = (a.astype(np.float64) for a in (q, k, v))
+    for h in range(n_heads):
+        sl = slice(h * 128, (h + 1) * 128)
+        sc = k64[:, sl] @ q64[0, sl] / np.sqrt(128.0)
+        p = np.exp(sc - sc.max())
+        p /= p.sum()
+        o = p @ v64[:, sl]
+        assert np.max(np.abs(got[0, sl].astype(np.float64) - o)) <= 4e-3 * max(np.max(np.abs(o)), 0.05)
+    if T == 1:
+        assert (got.view(np.uint16) == v[:1].view(np.uint16)).all()  # a single row has probability 1
+
+
+def test_softmax_logits_kernel_order():
+    for n, temp in ((32000, 0.8), (2048, 1.0), (8, 0.5)):
+        x = f16(RNG.normal(0, 1.3, n))
+        got = O.softmax_logits_kernel_order(x, temp)
+        ref = O.softmax_rows(x.reshape(1, -1), temp)[0]
+        # only the association of the sum differs: at most the last fp16 bit of a probability
+        d = np.abs(got.view(np.uint16).astype(np.int32) - ref.view(np.uint16).astype(np.int32))
+        assert d.max() <= 1 and (d != 0).mean() <= 0.02
+        assert abs(got.astype(np.float64).sum() - 1.0) <= 2e-3
+        assert np.argmax(got) == np.argmax(x)
 
 
 # ------------------------------------------------------------------ rms norm

@@ -13,8 +13,10 @@
  *   - every function returns 0 on success and a negative code on failure, never throws, never
  *     exits; lcu_last_error() describes the last failure of the calling thread
  *   - shapes the kernels do not support are rejected before any launch (LCU_E_SHAPE)
- *   - one host thread per stream; the library keeps no global mutable state besides per-device
- *     workspaces created by lcu_init
+ *   - one host thread per stream.  Operators that work in two launches keep partial results in
+ *     a 32 MiB workspace: every stream made by lcu_stream_create owns one (so contexts, which each
+ *     create a stream, never share scratch), the default stream and streams made elsewhere use one
+ *     per device created by lcu_init - calls on those that overlap on one device race
  */
 #ifndef LLAMA_CU_HIP_H
 #define LLAMA_CU_HIP_H
@@ -75,8 +77,7 @@ int lcu_event_elapsed_ms(float* out_ms, void* start_event, void* stop_event);   
  * (llama_cu.cu:1463-1496, 150-220, 225-285): M == 1 runs the streaming GEMV, larger M the MFMA
  * GEMM.  K must be a multiple of 8.  fp32 accumulation, one rounding to fp16 of acc + beta*out.
  * With 2 <= M <= 64 (short prompts) and K a multiple of 128 the K range is split over workgroups
- * and the fp32 partial sums pass through the per-device workspace (both GEMM entry points): such
- * calls that overlap on one device race. */
+ * and the fp32 partial sums pass through the stream's workspace (both GEMM entry points). */
 int lcu_gemm_f16_nt(void* out_dev, const void* lhs_dev, const void* rhs_dev, int M, int K, int N,
                     float beta, void* stream);
 /* lcu_gemm_f16u8_nt replaces matmul_nt(generic_tensor&) for quantised weights and
@@ -155,7 +156,7 @@ int lcu_attention(void* out_dev, const void* q_dev, const void* k_dev, const voi
  * when the kernel runs; max_T bounds it (at most the cache length; the position is clamped to it).
  * A bound of 1024 or less selects the single-launch kernel, a larger one the two-launch form that
  * spreads long rows over the chip, so a caller that replays a captured graph keeps the bound at
- * 1024 while the position allows it.  Uses the per-device workspace when max_T > 1024. */
+ * 1024 while the position allows it.  Uses the stream's workspace when max_T > 1024. */
 int lcu_attention_decode(void* out_dev, const void* q_dev, const void* k_dev, const void* v_dev,
                          const void* pos_dev, int max_T, int dim, int n_heads, void* stream);
 
@@ -226,7 +227,7 @@ int lcu_fill_f16(void* out_dev, size_t n, uint16_t bits, void* stream);
 /* error_stats, transform.cu:99-150 (launch site 175): out3 = {mean squared difference, largest
  * absolute difference, mean absolute difference} of two fp16 arrays of n elements, as fp32.
  * Deterministic (partials are added in index order, where the reference uses atomics).  Uses the
- * per-device workspace: calls that overlap on one device race. */
+ * stream's workspace. */
 int lcu_error_stats(void* out3_dev, const void* a_dev, const void* b_dev, size_t n, void* stream);
 
 #ifdef __cplusplus

@@ -268,13 +268,9 @@ __global__ __launch_bounds__(256) void dec_softmax_pv_kernel(half_t* __restrict_
   }
 }
 
-// scores scratch: n_heads x T_cap halves of the per-device workspace
+// scores: n_heads x T_cap halves of scratch (only touched when T_cap > SINGLE_LAUNCH_MAX_T)
 int launch_decode_attention(half_t* out, const half_t* q, const half_t* k, const half_t* v, const int* pos_dev,
-                            int T_cap, int dim, int n_heads, hipStream_t s) {
-  device_state* st = current_device_state();
-  if (!st || !st->ready) return set_error(LCU_E_NOINIT, "lcu_attention: lcu_init has not run on this device");
-  LCU_REQUIRE((size_t)n_heads * T_cap * sizeof(half_t) <= st->workspace_bytes, "lcu_attention: workspace too small");
-  half_t* scores = (half_t*)st->workspace;
+                            int T_cap, int dim, int n_heads, half_t* scores, hipStream_t s) {
   // up to 1024 cached rows the single launch wins (10.3 us against 11.0 us at T = 576: the second
   // launch costs more than the spreading saves), beyond that the two launches do (21 us against
   // 28 us at T = 2048)
@@ -518,8 +514,10 @@ int lcu_attention(void* out_dev, const void* q_dev, const void* k_dev, const voi
   hipStream_t s = as_stream(stream);
   if (n_new == 1) {
     LCU_REQUIRE(T <= MAX_T_DECODE, "lcu_attention: T %d exceeds %d", T, MAX_T_DECODE);
+    const workspace_t ws = workspace_for(s);
+    LCU_REQUIRE((size_t)n_heads * T * sizeof(half_t) <= ws.bytes, "lcu_attention: workspace too small");
     return launch_decode_attention((half_t*)out_dev, (const half_t*)q_dev, (const half_t*)k_dev, (const half_t*)v_dev,
-                                   nullptr, T, dim, n_heads, s);
+                                   nullptr, T, dim, n_heads, (half_t*)ws.ptr, s);
   }
   LCU_REQUIRE(T <= MAX_T_PREFILL, "lcu_attention: T %d exceeds %d for n_new > 1", T, MAX_T_PREFILL);
   // 16-row tiles when 32-row tiles would leave the grid under four workgroups per compute unit
@@ -560,8 +558,11 @@ int lcu_attention_decode(void* out_dev, const void* q_dev, const void* k_dev, co
               "lcu_attention_decode: dim %d / heads %d unsupported (head_dim must be 128, at most %d heads)", dim,
               n_heads, MAX_HEADS);
   LCU_REQUIRE(max_T > 0 && max_T <= MAX_T_DECODE, "lcu_attention_decode: max_T %d outside 1..%d", max_T, MAX_T_DECODE);
+  const workspace_t ws = workspace_for(as_stream(stream));
+  if (ws.ptr == nullptr) return set_error(LCU_E_NOINIT, "lcu_attention_decode: lcu_init has not run on this device");
+  LCU_REQUIRE((size_t)n_heads * max_T * sizeof(half_t) <= ws.bytes, "lcu_attention_decode: workspace too small");
   return launch_decode_attention((half_t*)out_dev, (const half_t*)q_dev, (const half_t*)k_dev, (const half_t*)v_dev,
-                                 (const int*)pos_dev, max_T, dim, n_heads, as_stream(stream));
+                                 (const int*)pos_dev, max_T, dim, n_heads, (half_t*)ws.ptr, as_stream(stream));
 }
 
 int lcu_attention_decode_batch(void* out_dev, const void* q_dev, const void* k_cache_ptrs_dev,

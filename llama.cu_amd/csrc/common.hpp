@@ -39,14 +39,25 @@ inline hipStream_t as_stream(void* s) { return reinterpret_cast<hipStream_t>(s);
 
 #define LCU_LAUNCH_CHECK() LCU_HIP(hipGetLastError())
 
-// per-device workspace created by lcu_init (attention partial results and counters)
+// per-device state created by lcu_init
 struct device_state {
   bool ready = false;
   int compute_units = 0;
-  void* workspace = nullptr;
+  void* workspace = nullptr;  // scratch of the default stream and of streams this library did not create
   size_t workspace_bytes = 0;
 };
 device_state* current_device_state();
+
+// Scratch memory for operators that work in two launches (partial sums of split-K products, scores
+// of long decode rows, partial error statistics).  Every stream made by lcu_stream_create owns a
+// workspace of its own, so that contexts driven from different host threads (each has its stream)
+// never share scratch; the default stream and foreign streams use the device's.  nullptr when
+// lcu_init has not run on the current device.
+struct workspace_t {
+  void* ptr = nullptr;
+  size_t bytes = 0;
+};
+workspace_t workspace_for(hipStream_t stream);
 
 // fp32 -> fp16, round to nearest even, as a separate step.  Written through an opaque register so
 // the compiler cannot merge the conversion into the preceding multiply or fused multiply-add

@@ -854,9 +854,9 @@ int lcu_fill_f16(void* out_dev, size_t n, uint16_t bits, void* stream) {
 
 int lcu_error_stats(void* out3_dev, const void* a_dev, const void* b_dev, size_t n, void* stream) {
   LCU_REQUIRE(out3_dev && a_dev && b_dev && n > 0, "lcu_error_stats: bad arguments");
-  device_state* st = current_device_state();
-  if (!st || !st->ready) return set_error(LCU_E_NOINIT, "lcu_error_stats: lcu_init has not run on this device");
-  float* partials = (float*)st->workspace;  // 256 x 3 floats of the per-device workspace
+  const workspace_t ws = workspace_for(as_stream(stream));
+  if (ws.ptr == nullptr) return set_error(LCU_E_NOINIT, "lcu_error_stats: lcu_init has not run on this device");
+  float* partials = (float*)ws.ptr;  // 256 x 3 floats of the stream's workspace
   error_stats_partial_kernel<<<ERR_BLOCKS, 256, 0, as_stream(stream)>>>(partials, (const half_t*)a_dev,
                                                                         (const half_t*)b_dev, n);
   LCU_LAUNCH_CHECK();

@@ -5,18 +5,21 @@
 // the natural operand order of v_mfma_f32_32x32x16_f16: every lane feeds 8 consecutive k of one
 // row of lhs (A) and of one row of W (B).
 //
-//   - 4 wavefronts in a 2x2 grid over the block tile BM x BN, K step 64; optionally a second
-//     such group in the same workgroup that takes the other half of a 128-wide K stage
-//   - global -> registers -> LDS with two LDS buffers and two register stages: while the matrix
-//     cores work on K step t, step t+1 waits in registers and step t+2 is being fetched; LDS rows
-//     are padded by 16 bytes so the 16-byte operand reads of 16 neighbouring lanes fall in
-//     distinct banks
-//   - the K loop carries no vector address arithmetic and no predication (see load_tile)
-//   - uint8 weights are dequantised between the global load and the LDS store, so each weight is
-//     converted once per block tile, to exactly fp16((q - 127.5) * scale) (287-289)
-//   - block index -> tile mapping keeps the tiles that share a slice of W on one XCD (one L2)
-//   - no padding rows: rows >= M and columns >= N are masked instead of the reference's zeroed
-//     "gutter" (llama_cu.h:236-242)
+// Two kernels:
+//   gemm_dl_kernel (K a multiple of 128, every shape of the model family): both operands travel
+//     from global memory straight into a ring of 2-3 LDS stages with global_load_lds_dwordx4 (no
+//     staging registers, no LDS store instructions); rows are unpadded and the 16-byte chunks of a
+//     row are permuted so that neither the requests nor the fragment reads meet in a bank; tiles
+//     of 256x128, 128x128 or 128x64 with 4 or 8 wavefronts (a second group of four may take the
+//     other half of a 128-wide K stage), chosen by how many tiles the product has; uint8 weights
+//     add a ring of codes and of scales and are turned into fp16 -- exactly fp16((q - 127.5) *
+//     scale), llama_cu.cu:287-289 -- once per block tile; with 2..64 rows the K range is split over
+//     workgroups and a second launch adds the fp32 partial sums (launch_skinny)
+//   gemm_kernel (ragged K): global -> registers -> padded LDS with two LDS buffers and two
+//     register stages, uint8 weights dequantised between the load and the LDS store
+// Both: the K loop carries no vector address arithmetic and no predication; the block index ->
+// tile mapping keeps the tiles that share a slice of W on one XCD (one L2); rows >= M and columns
+// >= N are masked instead of the reference's zeroed "gutter" rows (llama_cu.h:236-242).
 #include <type_traits>
 
 #include "common.hpp"
@@ -471,11 +474,11 @@ __global__ __launch_bounds__(64 * WM * WN * KS, WM * WN * KS <= 4 ? 2 : 1) void 
   const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char*)gemm_lds;
   auto request16 = [&](const void* g, uint32_t lds_off) {
     const uint32_t m0 = __builtin_amdgcn_readfirstlane(lds0 + lds_off);
-    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(g), "s"(m0) : "memory");
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(g), "s"(m0) : "memory", "m0");
   };
   auto request4 = [&](const void* g, uint32_t lds_off) {
     const uint32_t m0 = __builtin_amdgcn_readfirstlane(lds0 + lds_off);
-    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %0, off" ::"v"(g), "s"(m0) : "memory");
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %0, off" ::"v"(g), "s"(m0) : "memory", "m0");
   };
   // request `idx` (0 .. P-1) of this wavefront for batch `stage` into ring slot `slot`: the lhs tile
   // of that stage, and the W tile of that stage (fp16) or the codes and scales of the stage after it
@@ -828,7 +831,8 @@ int launch_skinny(operands_t op, const half_t* A, int M, int K, int N, int block
   static_assert(lds <= 160 * 1024, "LDS");
   *done = false;
   device_state* ds = current_device_state();
-  if (ds == nullptr || ds->workspace == nullptr) {
+  const workspace_t ws = workspace_for(st);
+  if (ds == nullptr || ws.ptr == nullptr) {
     return LCU_OK;
   }
   const int tiles_m = (M + BM - 1) / BM, tiles_n_per = (N + BN - 1) / BN, tiles_n = tiles_n_per * op.n_mats;
@@ -839,10 +843,10 @@ int launch_skinny(operands_t op, const half_t* A, int M, int K, int N, int block
   int splits = (ds->compute_units + tiles_m * tiles_n - 1) / (tiles_m * tiles_n);
   splits = max(1, min(splits, nt_all / 4));
   const size_t mn = (size_t)M * N;
-  while (splits > 1 && (size_t)splits * mn * op.n_mats * sizeof(float) > ds->workspace_bytes) {
+  while (splits > 1 && (size_t)splits * mn * op.n_mats * sizeof(float) > ws.bytes) {
     --splits;
   }
-  if ((size_t)splits * mn * op.n_mats * sizeof(float) > ds->workspace_bytes ||
+  if ((size_t)splits * mn * op.n_mats * sizeof(float) > ws.bytes ||
       (long)tiles_m * tiles_n * splits < ds->compute_units / 2) {
     return LCU_OK;
   }
@@ -856,7 +860,7 @@ int launch_skinny(operands_t op, const half_t* A, int M, int K, int N, int block
       raised[dev & 15] = true;
     }
   }
-  float* part = (float*)ds->workspace;
+  float* part = (float*)ws.ptr;
   kernel<<<tiles_m * tiles_n * splits, 256 * KS, lds, st>>>(op.out, A, op.W, op.S, M, K, N, block, beta, tiles_m, tiles_n,
                                                             part, splits, op.more);
   LCU_LAUNCH_CHECK();
@@ -872,13 +876,34 @@ int launch_skinny(operands_t op, const half_t* A, int M, int K, int N, int block
   return LCU_OK;
 }
 
+// The direct-to-LDS kernels fetch a thread's fp16 scale as the aligned 4-byte word that holds it:
+// every scale array must then start on a 4-byte boundary and hold an even number of scales (the
+// word of the last scale must not reach past the array).  Otherwise the register-staged kernel runs.
+template <bool U8>
+bool scale_words_ok(const operands_t& op, int K, int N, int block) {
+  if constexpr (!U8) {
+    return true;
+  } else {
+    if (((size_t)N * (size_t)(K / block)) % 2 != 0) {
+      return false;
+    }
+    const half_t* all[3] = {op.S, op.n_mats > 1 ? op.more.S[0] : nullptr, op.n_mats > 2 ? op.more.S[1] : nullptr};
+    for (const half_t* p : all) {
+      if (p != nullptr && (reinterpret_cast<uintptr_t>(p) & 3) != 0) {
+        return false;
+      }
+    }
+    return true;
+  }
+}
+
 // the split-K product of a few rows with its partial sums left in the workspace; *done = false when
 // the shape does not take that path (nothing has been launched then)
 template <bool U8>
 int skinny_partial(operands_t op, const half_t* A, int M, int K, int N, int block, hipStream_t st, bool* done,
                    partial_sums_t* res) {
   *done = false;
-  if (K % 128 != 0 || M > 64 || M < 1) {
+  if (K % 128 != 0 || M > 64 || M < 1 || !scale_words_ok<U8>(op, K, N, block)) {
     return LCU_OK;
   }
   if constexpr (U8) {
@@ -1081,7 +1106,8 @@ int dispatch_gemm(operands_t op, const half_t* A, int M, int K, int N, int block
   // unless each of them already fills the chip with 256x128 tiles and fusing saves no round of
   // workgroups (W1 + W3 at M = 512, N = 11008: 344 tiles take two rounds either way, and the fused
   // launch measured 132 us against 2 x 63 us).
-  if (op.n_mats > 1 && M > 64 && K % 128 == 0) {
+  const bool whole_stages = K % 128 == 0 && scale_words_ok<U8>(op, K, N, block);
+  if (op.n_mats > 1 && M > 64 && whole_stages) {
     device_state* ds = current_device_state();
     const long cus = ds && ds->compute_units > 0 ? ds->compute_units : 256;
     const long per = (long)((M + 255) / 256) * ((N + 127) / 128);
@@ -1100,7 +1126,7 @@ int dispatch_gemm(operands_t op, const half_t* A, int M, int K, int N, int block
   const long nm = op.n_mats;
   const long tiles128 = (long)((M + 127) / 128) * ((N + 127) / 128) * nm;
   const long tiles64 = (long)((M + 127) / 128) * ((N + 63) / 64) * nm;
-  if (K % 128 == 0 && M <= 64) {  // short prompts: the weight stream is what counts
+  if (whole_stages && M <= 64) {  // short prompts: the weight stream is what counts
     bool done = false;
     int rc;
     if constexpr (U8) {  // 64-row tiles with the code ring would leave LDS for one workgroup only
@@ -1113,7 +1139,7 @@ int dispatch_gemm(operands_t op, const half_t* A, int M, int K, int N, int block
       return rc;
     }
   }
-  if (K % 128 == 0) {  // whole stages: the direct-to-LDS kernels
+  if (whole_stages) {  // whole stages: the direct-to-LDS kernels
     const long tiles256 = (long)((M + 255) / 256) * ((N + 127) / 128) * nm;
     if (tiles256 >= 160) return launch_dl<256, 128, 4, 2, 1, 3, U8>(op, A, M, K, N, block, beta, st);
     if constexpr (!U8) {  // uint8 needs a code ring and two W tiles besides: too much LDS for two workgroups

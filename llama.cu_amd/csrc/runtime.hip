@@ -4,6 +4,9 @@
 #include <stdarg.h>
 #include <string.h>
 
+#include <mutex>
+#include <unordered_map>
+
 #include "common.hpp"
 
 namespace lcu {
@@ -17,6 +20,25 @@ int set_error(int code, const char* fmt, ...) {
   vsnprintf(g_error, sizeof(g_error), fmt, ap);
   va_end(ap);
   return code;
+}
+
+constexpr size_t WORKSPACE_BYTES = 32u << 20;
+static std::mutex g_stream_mutex;
+static std::unordered_map<hipStream_t, workspace_t> g_stream_workspaces;
+
+workspace_t workspace_for(hipStream_t stream) {
+  if (stream != nullptr) {
+    std::lock_guard<std::mutex> lock(g_stream_mutex);
+    auto it = g_stream_workspaces.find(stream);
+    if (it != g_stream_workspaces.end()) {
+      return it->second;
+    }
+  }
+  device_state* st = current_device_state();
+  if (st == nullptr || !st->ready) {
+    return workspace_t{};
+  }
+  return workspace_t{st->workspace, st->workspace_bytes};
 }
 
 device_state* current_device_state() {
@@ -49,10 +71,10 @@ int lcu_init(int device) {
                      device, prop.gcnArchName);
   }
   st.compute_units = prop.multiProcessorCount;
-  // per-device workspace for operators that work in two launches (lcu_error_stats: 256 x 3
-  // partial sums; decode attention over long rows: its scores; GEMMs with few rows: the fp32
-  // partial sums of their K splits); calls that use it and overlap on one device race
-  st.workspace_bytes = 32u << 20;
+  // workspace of the default stream for operators that work in two launches (lcu_error_stats:
+  // 256 x 3 partial sums; decode attention over long rows: its scores; GEMMs with few rows: the
+  // fp32 partial sums of their K splits); streams from lcu_stream_create bring their own
+  st.workspace_bytes = WORKSPACE_BYTES;
   LCU_HIP(hipMalloc(&st.workspace, st.workspace_bytes));
   LCU_HIP(hipMemset(st.workspace, 0, st.workspace_bytes));
   LCU_HIP(hipDeviceSynchronize());
@@ -137,13 +159,43 @@ int lcu_stream_create(void** out_stream) {
   LCU_REQUIRE(out_stream != nullptr, "lcu_stream_create: null output");
   hipStream_t s;
   LCU_HIP(hipStreamCreateWithFlags(&s, hipStreamNonBlocking));  // default priority
+  // the stream's own scratch, allocated here and not at first use: a first use may sit inside a
+  // graph capture, where nothing may be allocated
+  workspace_t ws;
+  ws.bytes = WORKSPACE_BYTES;
+  hipError_t e = hipMalloc(&ws.ptr, ws.bytes);
+  if (e == hipSuccess) {
+    e = hipMemset(ws.ptr, 0, ws.bytes);
+  }
+  if (e != hipSuccess) {
+    (void)hipFree(ws.ptr);
+    (void)hipStreamDestroy(s);
+    return set_error(LCU_E_HIP, "lcu_stream_create: workspace allocation failed: %s", hipGetErrorString(e));
+  }
+  {
+    std::lock_guard<std::mutex> lock(g_stream_mutex);
+    g_stream_workspaces[s] = ws;
+  }
   *out_stream = s;
   return LCU_OK;
 }
 
 int lcu_stream_destroy(void* stream) {
   if (stream) {
+    workspace_t ws;
+    {
+      std::lock_guard<std::mutex> lock(g_stream_mutex);
+      auto it = g_stream_workspaces.find(as_stream(stream));
+      if (it != g_stream_workspaces.end()) {
+        ws = it->second;
+        g_stream_workspaces.erase(it);
+      }
+    }
+    LCU_HIP(hipStreamSynchronize(as_stream(stream)));
     LCU_HIP(hipStreamDestroy(as_stream(stream)));
+    if (ws.ptr) {
+      LCU_HIP(hipFree(ws.ptr));
+    }
   }
   return LCU_OK;
 }

@@ -215,7 +215,9 @@ struct llama_batch_context_impl final : public llama_batch_context {
 
 /* static */ std::unique_ptr<llama_batch_context> llama_batch_context::create(llama_model* model, int n_sequences,
                                                                               int context_len, float temperature) {
-  if (model == nullptr || n_sequences < 1 || context_len < 1) {
+  if (model == nullptr || n_sequences < 1 || context_len < 1 || context_len > LLAMA_CU_MAX_CONTEXT) {
+    fprintf(stderr, "unsupported batch: %d sequences, context length %d (1..%d)\n", n_sequences, context_len,
+            LLAMA_CU_MAX_CONTEXT);
     return nullptr;
   }
   return std::make_unique<llama_batch_context_impl>(model, n_sequences, context_len, temperature);

@@ -166,7 +166,11 @@ lcu_context* lcu_context_create(lcu_model* m, int context_len, float temperature
   if (!m || context_len <= 0 || !(temperature > 0.0f)) {
     return nullptr;
   }
-  return new lcu_context{llama_context::create(m->model.get(), context_len, temperature)};
+  auto ctx = llama_context::create(m->model.get(), context_len, temperature);
+  if (!ctx) {
+    return nullptr;  // context length beyond what the attention kernels cover
+  }
+  return new lcu_context{std::move(ctx)};
 }
 
 void lcu_context_destroy(lcu_context* c) { delete c; }

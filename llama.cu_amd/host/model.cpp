@@ -178,6 +178,11 @@ static bool shapes_supported(llama_params const& p) {
     fprintf(stderr, "unsupported model shape: dim %u with %u heads (head_dim must be 128)\n", p.dim, p.n_heads);
     return false;
   }
+  if (p.n_heads > 64 || p.dim > 8192 || p.dim % 16 != 0 || p.ffn_dim() > 24576) {
+    fprintf(stderr, "unsupported model shape: dim %u (at most 8192), %u heads (at most 64), ffn %u (at most 24576)\n",
+            p.dim, p.n_heads, p.ffn_dim());
+    return false;
+  }
   if (p.n_vocab == 0 || p.n_vocab > 32767) {
     fprintf(stderr, "unsupported vocabulary size %u (token ids are 16-bit)\n", p.n_vocab);
     return false;
@@ -408,6 +413,22 @@ short llama_context_impl::next_token(std::vector<short> const& new_tokens) {
   const int n = (int)new_tokens.size();
   assert(n > 0);
   assert(new_tokens.size() + start_pos_ <= (size_t)context_len_);  // llama_cu.cu:1074
+  if (n > 1 && start_pos_ + n > LLAMA_CU_MAX_PREFILL_ROWS) {
+    // The multi-row attention kernel covers cache rows up to LLAMA_CU_MAX_PREFILL_ROWS: what fits
+    // below that goes in one call, every later token as a call of its own (same results: a row
+    // of a multi-row call and a one-row call compute the same thing, llama_cu.cu:1099-1186).
+    size_t done = 0;
+    short last = 0;
+    if (start_pos_ + 1 < LLAMA_CU_MAX_PREFILL_ROWS) {
+      done = (size_t)(LLAMA_CU_MAX_PREFILL_ROWS - start_pos_);
+      last = next_token(std::vector<short>(new_tokens.begin(), new_tokens.begin() + done));
+    }
+    for (; done < new_tokens.size(); ++done) {
+      last = next_token(std::vector<short>(1, new_tokens[done]));
+    }
+    last_n_ = 1;
+    return last;
+  }
   const int dim = p.dim, vocab = p.n_vocab;
   const int block = p.q_type == quantization_type::uint8 ? p.quantization_block_size : 0;
   char* x = (char*)t_embed_.data();
@@ -474,6 +495,12 @@ short llama_context_impl::next_token(std::vector<short> const& new_tokens) {
 
 /* static */ std::unique_ptr<llama_context> llama_context::create(llama_model* model, int context_len,
                                                                   float temperature) {
+  // The reference leaves context_len free (llama_cu.h:376); the attention kernels here hold a row of
+  // scores per head in LDS, which bounds it.  Refused at creation, not in the middle of a generation.
+  if (model == nullptr || context_len <= 0 || context_len > LLAMA_CU_MAX_CONTEXT) {
+    fprintf(stderr, "unsupported context length %d (1..%d)\n", context_len, LLAMA_CU_MAX_CONTEXT);
+    return nullptr;
+  }
   return std::make_unique<llama_context_impl>(model, context_len, temperature);
 }
 

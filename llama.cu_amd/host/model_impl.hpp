@@ -8,6 +8,12 @@
 
 namespace llama_cu {
 
+// limits of the attention kernels (csrc/attention.hip): cache rows a one-token call can attend to,
+// and cache rows a multi-token call can
+constexpr int LLAMA_CU_MAX_CONTEXT = 4096;
+constexpr int LLAMA_CU_MAX_PREFILL_ROWS = 2048;
+
+
 // one weight matrix [rows, cols]: fp16 values, or uint8 codes with fp16 scales [rows, cols/block]
 // (the reference's generic_tensor, llama_cu.h:252-270)
 struct weight_tensor {

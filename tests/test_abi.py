@@ -63,3 +63,18 @@ def test_reference_public_surface_compiles_and_links(tmp_path):
     res = subprocess.run(cmd, capture_output=True, text=True)
     assert res.returncode == 0, res.stderr
     assert exe.exists()
+
+
+def test_reference_main_program_compiles_against_the_kept_interface():
+    """The reference's own main.cpp, read from the reference checkout where that exists (it is not
+    copied here), is valid C++17 against include/llama_cu.h: same names, signatures and implicit
+    conversions as the reference's llama_cu.h."""
+    import shutil
+    import subprocess
+    src = "/root/reference/main.cpp"
+    if shutil.which("g++") is None or not os.path.exists(src):
+        pytest.skip("needs g++ and the reference checkout")
+    with open(src, "rb") as f:
+        res = subprocess.run(["g++", "-std=c++17", "-fsyntax-only", "-x", "c++", "-I", os.path.join(ROOT, "include"), "-"],
+                             stdin=f, capture_output=True, text=True)
+    assert res.returncode == 0, res.stderr

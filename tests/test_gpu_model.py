@@ -266,6 +266,47 @@ def test_context_api_behaviour(gpu):
     assert c.memory_usage() > 2 * 2 * 8 * 256 * 2
 
 
+def test_context_length_limits(gpu):
+    """The attention kernels bound the context length: a longer one is refused when the context is
+    created (the reference leaves it free, llama_cu.h:376), never in the middle of a generation."""
+    G = gpu
+    gm = G.P.Model(**TINY, seed=1)
+    with pytest.raises(G.P.LcuError):
+        G.P.Context(gm, context_len=4097, temperature=0.8)
+    with pytest.raises(G.P.LcuError):
+        G.P.BatchContext(gm, 2, context_len=8192, temperature=0.8)
+    c = G.P.Context(gm, context_len=4096, temperature=0.8)
+    assert c.tokens_left() == 4096
+    c.close()
+    gm.close()
+
+
+def test_prompt_longer_than_the_multi_row_attention_reaches(gpu):
+    """A multi-token call that ends beyond 2048 cache rows is served in pieces (rows up to 2048 in one
+    call, the rest one token at a time) and gives what the oracle gives for the whole call."""
+    G = gpu
+    cfg = dict(dim=256, multiple_of=128, n_heads=2, n_layers=1, n_vocab=320)
+    om = O.Model(**cfg, seed=9, weight_std=0.05)
+    gm = G.P.Model(**cfg, seed=9, weight_std=0.05)
+    oc = O.Context(om, context_len=2200, temperature=0.8)
+    gc = G.P.Context(gm, context_len=2200, temperature=0.8)
+    toks = np.random.default_rng(4).integers(0, cfg["n_vocab"], 2199).astype(np.int16)
+    otok, _, ologits, _ = oc.next_token(toks[:2100], want=True)
+    gtok = gc.next_token(toks[:2100])
+    assert gc.tokens_left() == 100
+    assert G.max_abs_rel(gc.logits(), ologits) <= TOL
+    # a second multi-token call that starts beyond the limit: all of it goes token by token
+    otok, _, ologits, _ = oc.next_token(toks[2100:2150], want=True)
+    gtok = gc.next_token(toks[2100:2150])
+    assert gc.tokens_left() == 50
+    assert G.max_abs_rel(gc.logits(), ologits) <= TOL
+    ok, ov = oc.kv(0, 2150)
+    gk, gv = gc.kv(0, 2150)
+    assert G.max_abs_rel(gk, ok) <= TOL and G.max_abs_rel(gv, ov) <= TOL
+    gc.close()
+    gm.close()
+
+
 def test_sampling_follows_the_step_random_sequence(gpu):
     # llama_context::sample_with_seed: token k is the oracle's draw from the probabilities of step k
     # with output k of splitmix64(seed); covers the eager step, the captured graph and its replays

@@ -275,6 +275,46 @@ def test_gemm_multi_matches_separate_calls(gpu, M, K, N, count):
     G.release()
 
 
+def test_streams_own_their_workspace(gpu):
+    """Split-K products (2..64 rows) keep fp32 partial sums in scratch memory.  Every stream made by
+    lcu_stream_create has a workspace of its own, so two host threads driving two streams at once
+    get the results of a single undisturbed call, bit for bit."""
+    import ctypes as C
+    import threading
+    G = gpu
+    L = G.L()
+    K, N = 4096, 4096
+    cases = []
+    for t in range(2):
+        x = normal((8 + 8 * t, K), 3, 40 + t, 1.0)
+        w = normal((N, K), 3, 50 + t, 0.02)
+        cases.append((x, w, G.gemm_f16(x, w)))
+    G.release()
+    results = [None, None]
+
+    def work(t):
+        x, w, _ = cases[t]
+        stream = G.B.vp()
+        G.B.check(L.lcu_stream_create(C.byref(stream)))
+        xd, wd, od = G.dev(x), G.dev(w), G.empty((x.shape[0], N))
+        bad = 0
+        for _ in range(200):
+            G.B.check(L.lcu_gemm_f16_nt(od.ptr, xd.ptr, wd.ptr, x.shape[0], K, N, 0.0, stream))
+        G.B.check(L.lcu_sync(stream))
+        results[t] = G.host(od, (x.shape[0], N))
+        G.B.check(L.lcu_stream_destroy(stream))
+        for b in (xd, wd, od):
+            b.free()
+
+    threads = [threading.Thread(target=work, args=(t,)) for t in range(2)]
+    for th in threads:
+        th.start()
+    for th in threads:
+        th.join()
+    for t in range(2):
+        assert results[t] is not None and (results[t].view(np.uint16) == cases[t][2].view(np.uint16)).all()
+
+
 def test_gemm_rejects_bad_shapes(gpu):
     G = gpu
     a = G.dev(np.zeros((4, 12), dtype=np.float16))

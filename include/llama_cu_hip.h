@@ -169,6 +169,16 @@ int lcu_attention_decode(void* out_dev, const void* q_dev, const void* k_dev, co
 int lcu_rope_store_batch(void* q_dev, const void* k_new_dev, const void* v_new_dev, const void* k_cache_ptrs_dev,
                          const void* v_cache_ptrs_dev, const void* pos_dev, int n_seq, int dim, int n_heads,
                          const void* table_dev, int table_positions, void* stream);
+/* lcu_attention for one new token (n_new == 1, T cached rows, start_pos = T - 1) that allocates
+ * nothing and touches no workspace: no counterpart in the reference; for callers that cannot
+ * call hipMalloc (code under HIP graph capture, serving loops and harnesses that forbid it).  The
+ * scores of rows longer than 1024 go through a static device array of 64 heads x 4096 rows of
+ * fp16 (512 KiB per GPU, held until the process ends): T beyond 4096 or more than 64 heads are
+ * rejected (LCU_E_SHAPE), lcu_init must have run on the current device (LCU_E_NOINIT).  Same bits
+ * as lcu_attention.  Every call on a GPU uses that GPU's one array: calls that overlap on one GPU
+ * (two streams, two threads) race. */
+int lcu_attention_decode_static(void* out_dev, const void* q_dev, const void* k_dev, const void* v_dev, int T,
+                                int dim, int n_heads, void* stream);
 /* lcu_attention_decode for every sequence in one launch: row b of q against rows 0..pos[b] of
  * sequence b's caches -> row b of out; max_T bounds pos[b] + 1 */
 int lcu_attention_decode_batch(void* out_dev, const void* q_dev, const void* k_cache_ptrs_dev,

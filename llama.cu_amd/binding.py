@@ -55,6 +55,7 @@ SIGNATURES = {
     "lcu_softmax_rows": (i32, [vp, vp, i32, i32, f32, vp]),
     "lcu_silu_mul": (i32, [vp, vp, vp, sz, vp]),
     "lcu_exp_f32": (i32, [vp, vp, sz, vp]),
+    "lcu_attention_decode_static": (i32, [vp, vp, vp, vp, i32, i32, i32, vp]),
     "lcu_embed": (i32, [vp, vp, i32, i32, vp, i32, vp]),
     "lcu_embed_u8": (i32, [vp, vp, i32, i32, vp, vp, i32, i32, vp]),
     "lcu_argmax_f16": (i32, [vp, vp, i32, vp]),

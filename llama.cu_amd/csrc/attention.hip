@@ -491,12 +491,39 @@ __global__ __launch_bounds__(256) void prefill_attention_kernel(half_t* __restri
   }
 }
 
+// ---- scores of long decode rows for callers that may not allocate --------------------------------
+// lcu_attention_decode_static keeps the fp16 scores of dec_scores_kernel in this array instead of
+// a workspace from hipMalloc: MAX_HEADS x MAX_T_DECODE halves = 512 KiB per GPU, held until the
+// process ends.  In host code the name `scratch` is only a handle: the array's device address is
+// fetched once per device with hipGetSymbolAddress (attention_static_init, called by lcu_init
+// with that device current) and kept in scratch_dev; kernels and host code use that pointer.
+constexpr int STATIC_MAX_DEVICES = 16;
+static __device__ __align__(256) half_t scratch[MAX_HEADS * MAX_T_DECODE];
+static half_t* scratch_dev[STATIC_MAX_DEVICES] = {};
+
 size_t prefill_lds_bytes(int BR, int Tc) {
   const size_t kv = (size_t)CW * QLD;
   return ((size_t)BR * QLD + kv + (size_t)BR * (Tc + 8)) * sizeof(half_t);
 }
 
 }  // namespace
+
+namespace lcu {
+
+// called by lcu_init with `device` current: the address of this device's copy of `scratch`
+int attention_static_init(int device) {
+  if (device < 0 || device >= STATIC_MAX_DEVICES) {
+    return set_error(LCU_E_SHAPE, "attention_static_init: device %d out of range", device);
+  }
+  if (scratch_dev[device] == nullptr) {
+    void* p = nullptr;
+    LCU_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+    scratch_dev[device] = (half_t*)p;
+  }
+  return LCU_OK;
+}
+
+}  // namespace lcu
 
 extern "C" {
 
@@ -563,6 +590,26 @@ int lcu_attention_decode(void* out_dev, const void* q_dev, const void* k_dev, co
   LCU_REQUIRE((size_t)n_heads * max_T * sizeof(half_t) <= ws.bytes, "lcu_attention_decode: workspace too small");
   return launch_decode_attention((half_t*)out_dev, (const half_t*)q_dev, (const half_t*)k_dev, (const half_t*)v_dev,
                                  (const int*)pos_dev, max_T, dim, n_heads, (half_t*)ws.ptr, as_stream(stream));
+}
+
+int lcu_attention_decode_static(void* out_dev, const void* q_dev, const void* k_dev, const void* v_dev, int T, int dim,
+                                int n_heads, void* stream) {
+  LCU_REQUIRE(out_dev && q_dev && k_dev && v_dev, "lcu_attention_decode_static: null pointer");
+  LCU_REQUIRE(n_heads > 0 && n_heads <= MAX_HEADS && dim == n_heads * HD,
+              "lcu_attention_decode_static: dim %d / heads %d unsupported (head_dim must be 128, at most %d heads)",
+              dim, n_heads, MAX_HEADS);
+  LCU_REQUIRE(T > 0 && T <= MAX_T_DECODE,
+              "lcu_attention_decode_static: %d cached rows, the static scores array holds rows of 1..%d", T,
+              MAX_T_DECODE);
+  int dev = 0;
+  LCU_HIP(hipGetDevice(&dev));
+  if (dev < 0 || dev >= STATIC_MAX_DEVICES || scratch_dev[dev] == nullptr) {
+    return set_error(LCU_E_NOINIT, "lcu_attention_decode_static: lcu_init has not run on device %d", dev);
+  }
+  // n_heads * T <= MAX_HEADS * MAX_T_DECODE halves by the checks above; every score a launch reads
+  // it has written itself, so nothing needs clearing between calls
+  return launch_decode_attention((half_t*)out_dev, (const half_t*)q_dev, (const half_t*)k_dev, (const half_t*)v_dev,
+                                 nullptr, T, dim, n_heads, scratch_dev[dev], as_stream(stream));
 }
 
 int lcu_attention_decode_batch(void* out_dev, const void* q_dev, const void* k_cache_ptrs_dev,

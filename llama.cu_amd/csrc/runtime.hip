@@ -11,6 +11,8 @@
 
 namespace lcu {
 
+int attention_static_init(int device);  // attention.hip
+
 static thread_local char g_error[512] = "";
 static device_state g_devices[16];
 
@@ -78,6 +80,10 @@ int lcu_init(int device) {
   LCU_HIP(hipMalloc(&st.workspace, st.workspace_bytes));
   LCU_HIP(hipMemset(st.workspace, 0, st.workspace_bytes));
   LCU_HIP(hipDeviceSynchronize());
+  const int rc = attention_static_init(device);
+  if (rc != LCU_OK) {
+    return rc;
+  }
   st.ready = true;
   return LCU_OK;
 }

@@ -9,10 +9,13 @@ read-back) after a 512-token prompt; weights are seeded random values of the mod
   value        tokens/s over exactly K timed steps (inputs and weights resident in HBM)
   roofline     the dominant decode kernel (W1/W3 GEMV + SiLU*mul of one layer, on an already
                normalised row) launched back to back over the model's own layers, timed with HIP
-               events on its stream: algorithmic bytes per launch / average launch time, against 8 TB/s
+               events on its stream: algorithmic bytes per launch / average launch time, against 8 TB/s;
+               whole_step_* in the same object is the quantity the decode target is stated in: all
+               bytes a decode step must read (weights + KV cache) / the measured step time
   cpu_baseline the CPU oracle (a port of the reference's arithmetic, OpenMP) decoding on the host
                cores on a bounded sample, extrapolated to the full depth; reported only
-  extra        per-shape GEMV GB/s, prefill GEMM TFLOP/s and prefill time measured in the same run
+  extra        per-shape GEMV GB/s, prefill GEMM TFLOP/s and prefill time measured in the same run,
+               and the other model of the metric (LLaMA-30B shape, uint8 weights) decoded the same way
 """
 import argparse
 import ctypes as C
@@ -245,14 +248,15 @@ def gemm_leg(P, stream):
 
 
 def cpu_baseline_leg(cfg):
-    """The CPU oracle (the checker, here only as the reported baseline) on a 2-layer slice of the
-    same model shape: per-layer and head costs measured, then extrapolated to the full depth."""
+    """The CPU oracle (the checker, here only as the reported baseline) on 2- and 6-layer slices of
+    the same model shape: per-layer and head costs measured, then extrapolated to the full depth."""
     sys.path.insert(0, os.path.join(ROOT, "tests"))
     import oracle_lib as O
     small = dict(cfg)
-    small["n_layers"] = 2
+    deep, shallow = (6, 2) if cfg["dim"] <= 4096 else (3, 1)
+    small["n_layers"] = deep
     m2 = O.Model(norm_eps=1e-6, qblock=128, seed=0, weight_std=0.02, **small)
-    small["n_layers"] = 1
+    small["n_layers"] = shallow
     m1 = O.Model(norm_eps=1e-6, qblock=128, seed=0, weight_std=0.02, **small)
     prompt = np.random.default_rng(0).integers(0, cfg["n_vocab"], PROMPT).astype(np.int16)
     times = []
@@ -266,14 +270,14 @@ def cpu_baseline_leg(cfg):
             tok = c.next_token([tok])
         times.append((time.perf_counter() - t0) / steps)
         c.close()
-    per_layer = max(times[1] - times[0], 1e-9)
-    head = max(times[0] - per_layer, 0.0)
+    per_layer = max((times[1] - times[0]) / (deep - shallow), 1e-9)
+    head = max(times[0] - per_layer * shallow, 0.0)
     full = head + per_layer * cfg["n_layers"]
     cores = O.lib().orc_num_threads()
     return dict(value=round(1.0 / full, 3), unit="tok/s", cores=int(cores), kind="port",
-                sample="CPU oracle decode at T~%d on 1- and 2-layer models of the same shape, %d steps each; "
+                sample="CPU oracle decode at T~%d on %d- and %d-layer models of the same shape, %d steps each; "
                        "per-layer %.1f ms and embedding+logits %.1f ms extrapolated to %d layers"
-                       % (PROMPT + 2, steps, per_layer * 1e3, head * 1e3, cfg["n_layers"]))
+                       % (PROMPT + 2, shallow, deep, steps, per_layer * 1e3, head * 1e3, cfg["n_layers"]))
 
 
 def batched_leg(P, model, cfg, sizes=(8, 32), prompt=64, steps=32, warmup=4):
@@ -327,7 +331,18 @@ def main():
     ctx.close()
     if not args.no_extra and not args.no_batched:
         extra["batched_decode"] = batched_leg(P, model, cfg)
+    ffn = model.ffn
     model.close()
+    if not args.no_extra and args.workload == "llama7b_fp16":
+        # the other model the metric names: LLaMA-30B shape with uint8 weights, decoded the same way
+        cfg30 = WORKLOADS["llama30b_u8"]
+        m30, c30, d30 = decode_leg(P, cfg30, args.steps, args.warmup)
+        extra["llama30b_u8"] = dict(tok_s=round(d30["tok_s"], 2), ms_per_step=round(d30["ms_per_step"], 4),
+                                    prefill_512_ms=round(d30["prefill_ms"], 3),
+                                    decode_bytes_per_token=int(d30["bytes_per_token"]),
+                                    frac=round(d30["bytes_per_token"] / d30["ms_per_step"] / 1e6 / HBM_PEAK_GBS, 3))
+        c30.close()
+        m30.close()
     if args.copy_calibration:
         n = 256 << 20
         a, b = B.DeviceBuffer(n), B.DeviceBuffer(n)
@@ -352,8 +367,10 @@ def main():
                                % (args.workload, PROMPT), "device": props.name.decode(errors="replace")},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC.get(args.workload),
-                     "kernel": "decode_ffn_up_kernel (W1,W3 GEMV + SiLU*mul), dim %d ffn %d" % (cfg["dim"], model.ffn),
-                     "bytes_per_launch": int(k_bytes), "us_per_launch": round(k_us, 3)},
+                     "kernel": "decode_ffn_up_kernel (W1,W3 GEMV + SiLU*mul), dim %d ffn %d" % (cfg["dim"], ffn),
+                     "bytes_per_launch": int(k_bytes), "us_per_launch": round(k_us, 3),
+                     "whole_step_achieved": extra["decode_hbm_gb_s"],
+                     "whole_step_frac": extra["decode_frac_of_hbm_roofline"]},
         "cpu_baseline": cpu,
         "extra": extra,
     }

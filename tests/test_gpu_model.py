@@ -399,22 +399,22 @@ def test_one_llama7b_layer_prefill_512_then_decode_at_2048(gpu):
     assert G.max_abs_rel(gk, ok) <= TOL and G.max_abs_rel(gv, ov) <= TOL
 
 
-# Greedy decoding compares argmax results, and an argmax is discontinuous: where the oracle's two
-# largest fp16 logits are within a few fp16 ulps of each other (logits of 4..8 have an ulp of
-# 0.0039), any other correct fp32-accumulating implementation -- the reference's own matmul_type 1
-# versus 4 included -- may order them the other way.  So every step must reproduce the oracle's
-# token, except at steps whose oracle margin is at most NEAR_TIE, where the device must still pick
-# one of the oracle's two candidates.  Steps are compared under teacher forcing (the oracle's token
-# is fed back), so one near-tie cannot hide the steps after it.
-#
-# How near is near depends on the depth of the model: rounding differences grow through the layers.
-# LLaMA-7B (32 layers): device and oracle logits differ by 0.006 on average, 0.02 at most, over the
-# fixture's steps.  LLaMA-30B (60 layers): 0.018 on average, 0.07 at most -- and the device's own
-# uint8 kernels differ by just as much from its fp16 kernels run on the dequantised weight values
-# (test_u8_and_f16_kernels_agree_at_30b_depth), so that figure is the noise floor of the depth, not
-# an error of one path.  An argmax can flip when the margin is below about twice the per-logit
-# deviation.
-NEAR_TIE = {"llama7b_fp16_seed0_greedy.json": 0.02, "llama30b_u8_seed0_greedy.json": 0.1}
+# Greedy decoding, teacher-forced (the oracle's token is fed back, so one differing step cannot hide
+# the steps after it).  The fixtures come from the oracle's flavour 2, which restates the summation
+# order of every kernel of a one-token step: with fp16 weights a decode step given the same cache is
+# the oracle's bit for bit (test_decode_steps_bit_exact_against_kernel_order_oracle).  What is left
+# between device and oracle is the 512-token prompt, whose products run on the matrix cores in an
+# order the hardware fixes (as the reference's own tensor cores do): the cached K and V of the
+# prompt differ in the last fp16 bit here and there, and the logits of later steps by a few fp16
+# ulps (an ulp is 0.0039 for logits of 4..8).  An argmax can only follow that where the oracle's two
+# best logits are closer than the deviation, so: every step must give the oracle's token, except
+# steps whose oracle margin is at most NEAR_TIE, where the device must still pick one of the
+# oracle's two candidates.  The measured deviation of the device's logits from the oracle's (on the
+# two best tokens of every step) is printed and bounded by DEVIATION.  With uint8 weights
+# v_dot2_f32_f16 adds three addends in a way of its own, which the oracle does not restate: a few
+# outputs in a thousand of every GEMV differ by one ulp, hence the wider bounds.
+NEAR_TIE = {"llama7b_fp16_seed0_greedy.json": 0.0079, "llama30b_u8_seed0_greedy.json": 0.03}
+DEVIATION = {"llama7b_fp16_seed0_greedy.json": 0.02, "llama30b_u8_seed0_greedy.json": 0.06}
 
 
 def greedy_case(G, name):
@@ -427,10 +427,12 @@ def greedy_case(G, name):
                    seed=fx["seed"], weight_std=fx["weight_std"])
     gc = G.P.Context(gm, context_len=fx["context_len"], temperature=fx["temperature"])
     feed = np.array(fx["prompt"], dtype=np.int16)
-    identical, near_ties, failures = 0, [], []
+    identical, near_ties, failures, dev = 0, [], [], []
     for step, want in enumerate(fx["tokens"]):
         tok = gc.next_token(feed)
         l1, l2, _, _ = fx["top2_logits_probs"][step]
+        got = gc.logits().astype(np.float64)
+        dev.append(max(abs(got[fx["top2_ids"][step][0]] - l1), abs(got[fx["top2_ids"][step][1]] - l2)))
         if tok == want:
             identical += 1
         elif l1 - l2 <= NEAR_TIE[name] and tok in fx["top2_ids"][step]:
@@ -441,8 +443,10 @@ def greedy_case(G, name):
         feed = np.array([want], dtype=np.int16)
     gc.close()
     gm.close()
-    print("%s: %d of %d steps identical; near-tie steps: %s" % (name, identical, len(fx["tokens"]), near_ties or "none"))
+    print("%s: %d of %d steps identical; near-tie steps: %s; deviation of the two best logits from the oracle's: "
+          "mean %.5f, max %.5f" % (name, identical, len(fx["tokens"]), near_ties or "none", np.mean(dev), np.max(dev)))
     n_close = sum(1 for t in fx["top2_logits_probs"] if t[0] - t[1] <= NEAR_TIE[name])
+    assert np.max(dev) <= DEVIATION[name]
     return identical, len(fx["tokens"]), near_ties, failures, n_close
 
 
@@ -451,7 +455,6 @@ def test_greedy_tokens_llama7b_fp16(gpu):
     identical, total, near_ties, failures, n_close = greedy_case(gpu, "llama7b_fp16_seed0_greedy.json")
     assert not failures, "\n".join(failures)
     assert identical + len(near_ties) == total and len(near_ties) <= n_close
-    assert identical >= total - 4
 
 
 def test_greedy_tokens_llama30b_u8(gpu):
@@ -459,7 +462,6 @@ def test_greedy_tokens_llama30b_u8(gpu):
     identical, total, near_ties, failures, n_close = greedy_case(gpu, "llama30b_u8_seed0_greedy.json")
     assert not failures, "\n".join(failures)
     assert identical + len(near_ties) == total and len(near_ties) <= n_close
-    assert identical >= total - 8
 
 
 def test_u8_and_f16_kernels_agree_at_30b_depth(gpu):

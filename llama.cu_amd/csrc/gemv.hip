@@ -119,17 +119,23 @@ struct batch_t {
   // Loads are unconditional: a chunk past the end of K is read from the last in-range position
   // instead (a predicated load becomes a branch, and the waits the compiler puts around branches
   // serialise the loads); fma() gives such a chunk a zero x.
+  // block_shift: log2 of the quantisation block when that is a power of two (a shift instead of
+  // the dozen instructions of an integer division per load), else -1
   __device__ __forceinline__ void load(const uint8_t* const (&rows)[R], const half_t* const (&srow)[R],
                                        const half_t* __restrict__ x, const half_t* __restrict__ norm_w, int kb, int K,
-                                       int block, int lane) {
+                                       int block, int block_shift, int lane) {
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const int kk = min((kb * U + u) * CHUNK + lane * VEC, K - VEC);
+      int sidx = 0;
+      if constexpr (U8) {
+        sidx = block_shift >= 0 ? kk >> block_shift : kk / block;
+      }
 #pragma unroll
       for (int r = 0; r < R; ++r) {
         w[u][r] = __builtin_nontemporal_load(reinterpret_cast<const uint4_t*>(rows[r] + (size_t)kk * (U8 ? 1 : 2)));
         if constexpr (U8) {
-          sc[u][r] = srow[r][kk / block];
+          sc[u][r] = srow[r][sidx];
         }
       }
 #pragma unroll
@@ -143,61 +149,64 @@ struct batch_t {
     }
   }
 
-  // xs: raw x in LDS (NORM only); kb, K, lane as in load()
+  // xs: raw x in LDS (NORM only); kb, K, lane as in load().  A piece past the end of K (its load
+  // was redirected to the last in-range position) is skipped: per wavefront when the whole chunk
+  // lies past K, per lane otherwise.
   __device__ __forceinline__ void fma(const half_t* xs, float rms_inv, int kb, int K, int lane, float (&a0)[R],
                                       float (&a1)[R]) const {
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-      half8_t xv[XV];
-#pragma unroll
-      for (int j = 0; j < XV; ++j) {
-        const int kk = (kb * U + u) * CHUNK + lane * VEC;
-        if constexpr (NORM) {
-          const half8_t raw = kk < K ? *reinterpret_cast<const half8_t*>(xs + kk + 8 * j) : (half8_t)(0.0f);
-          xv[j] = normed(raw, nw[u][j], rms_inv);
-        } else {
-          xv[j] = kk < K ? xr[u][j] : (half8_t)(0.0f);
-        }
+      const int kk = (kb * U + u) * CHUNK + lane * VEC;
+      if ((kb * U + u) * CHUNK >= K) {
+        continue;
       }
+      if (kk < K) {
+        half8_t xv[XV];
 #pragma unroll
-      for (int r = 0; r < R; ++r) {
-        if constexpr (U8) {
-          const half_t sv = sc[u][r];
-          const half_t hv = sv * (half_t)0.5f;
-          if (hv + hv == sv) {  // s/2 exact (every normal scale): 3-operation dequantisation
-            const half2_t s1v = {sv, sv}, h1v = {hv, hv};
+        for (int j = 0; j < XV; ++j) {
+          if constexpr (NORM) {
+            xv[j] = normed(*reinterpret_cast<const half8_t*>(xs + kk + 8 * j), nw[u][j], rms_inv);
+          } else {
+            xv[j] = xr[u][j];
+          }
+        }
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-              // selector bytes 4..7 pick from the first operand (0x64 in every byte), 0..3 from the codes
-              const half2_t lo = dequant2_fma(__builtin_amdgcn_perm(0x64646464u, w[u][r][j], 0x04010400u), s1v, h1v);
-              const half2_t hi = dequant2_fma(__builtin_amdgcn_perm(0x64646464u, w[u][r][j], 0x04030402u), s1v, h1v);
-              const half8_t& x8 = xv[j >> 1];
-              const int e = (j & 1) * 4;
-              const half2_t xlo = {x8[e], x8[e + 1]}, xhi = {x8[e + 2], x8[e + 3]};
-              a0[r] = __builtin_amdgcn_fdot2(lo, xlo, a0[r], false);
-              a1[r] = __builtin_amdgcn_fdot2(hi, xhi, a1[r], false);
+        for (int r = 0; r < R; ++r) {
+          if constexpr (U8) {
+            // 16 codes as four words; x as eight words of two halves.  Codes 0,1 of a word go with
+            // x word 2j into a0, codes 2,3 with x word 2j + 1 into a1 (v_dot2_f32_f16).
+            const uint4_t xw0 = __builtin_bit_cast(uint4_t, xv[0]), xw1 = __builtin_bit_cast(uint4_t, xv[XV - 1]);
+            const uint32_t xw[8] = {xw0[0], xw0[1], xw0[2], xw0[3], xw1[0], xw1[1], xw1[2], xw1[3]};
+            const half_t sv = sc[u][r];
+            const half_t hv = sv * (half_t)0.5f;
+            if (hv + hv == sv) {  // s/2 exact (every normal scale): 3-operation dequantisation
+              const half2_t s1v = {sv, sv}, h1v = {hv, hv};
+#pragma unroll
+              for (int j = 0; j < 4; ++j) {
+                // selector bytes 4..7 pick from the first operand (0x64 in every byte), 0..3 from the codes
+                const half2_t lo = dequant2_fma(__builtin_amdgcn_perm(0x64646464u, w[u][r][j], 0x04010400u), s1v, h1v);
+                const half2_t hi = dequant2_fma(__builtin_amdgcn_perm(0x64646464u, w[u][r][j], 0x04030402u), s1v, h1v);
+                a0[r] = __builtin_amdgcn_fdot2(lo, __builtin_bit_cast(half2_t, xw[2 * j]), a0[r], false);
+                a1[r] = __builtin_amdgcn_fdot2(hi, __builtin_bit_cast(half2_t, xw[2 * j + 1]), a1[r], false);
+              }
+            } else {  // a subnormal scale with an odd last bit: the four-operation form, same products
+              const half_t s2 = sv * (half_t)2.0f;  // exact
+              const half2_t s2v = {s2, s2};
+#pragma unroll
+              for (int j = 0; j < 4; ++j) {
+                const half2_t lo = dequant2(__builtin_amdgcn_perm(0u, w[u][r][j], 0x0c010c00u), s2v);
+                const half2_t hi = dequant2(__builtin_amdgcn_perm(0u, w[u][r][j], 0x0c030c02u), s2v);
+                a0[r] = __builtin_amdgcn_fdot2(lo, __builtin_bit_cast(half2_t, xw[2 * j]), a0[r], false);
+                a1[r] = __builtin_amdgcn_fdot2(hi, __builtin_bit_cast(half2_t, xw[2 * j + 1]), a1[r], false);
+              }
             }
           } else {
-            const half_t s2 = sv * (half_t)2.0f;  // exact
-            const half2_t s2v = {s2, s2};
+            const half8_t wv = __builtin_bit_cast(half8_t, w[u][r]);
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-              const half2_t lo = dequant2(__builtin_amdgcn_perm(0u, w[u][r][j], 0x0c010c00u), s2v);
-              const half2_t hi = dequant2(__builtin_amdgcn_perm(0u, w[u][r][j], 0x0c030c02u), s2v);
-              const half8_t& x8 = xv[j >> 1];
-              const int e = (j & 1) * 4;
-              a0[r] = fmaf((float)lo.x, (float)x8[e], a0[r]);
-              a1[r] = fmaf((float)lo.y, (float)x8[e + 1], a1[r]);
-              a0[r] = fmaf((float)hi.x, (float)x8[e + 2], a0[r]);
-              a1[r] = fmaf((float)hi.y, (float)x8[e + 3], a1[r]);
+            for (int e = 0; e < 8; e += 2) {
+              a0[r] = fmaf((float)wv[e], (float)xv[0][e], a0[r]);
+              a1[r] = fmaf((float)wv[e + 1], (float)xv[0][e + 1], a1[r]);
             }
-          }
-        } else {
-          const half8_t wv = __builtin_bit_cast(half8_t, w[u][r]);
-#pragma unroll
-          for (int e = 0; e < 8; e += 2) {
-            a0[r] = fmaf((float)wv[e], (float)xv[0][e], a0[r]);
-            a1[r] = fmaf((float)wv[e + 1], (float)xv[0][e + 1], a1[r]);
           }
         }
       }
@@ -219,19 +228,21 @@ struct stream_t {
   const Tasks tk;  // by value: a reference member kept the struct in scratch memory in some instantiations
   const half_t* x;
   const half_t* norm_w;
-  int K, block, lane, wave, task, n_batches;
+  int K, block, block_shift, lane, wave, task, n_batches;
   const uint8_t* rows[R];
   const half_t* srow[R];
   batch cur;
 
   __device__ __forceinline__ stream_t(const Tasks& t, const half_t* x_, const half_t* norm_w_, int K_, int block_,
                                       int task_)
-      : tk(t), x(x_), norm_w(norm_w_), K(K_), block(block_), lane(threadIdx.x & 63), wave(threadIdx.x >> 6),
+      : tk(t), x(x_), norm_w(norm_w_), K(K_), block(block_),
+        block_shift(block_ > 0 && (block_ & (block_ - 1)) == 0 ? __builtin_ctz(block_) : -1), lane(threadIdx.x & 63),
+        wave(threadIdx.x >> 6),
         task(task_), n_batches((K_ + batch::CHUNK * U * GEMV_WAVES - 1) / (batch::CHUNK * U * GEMV_WAVES)) {}
 
   __device__ __forceinline__ void begin() {
     tk.rows(task, rows, srow);
-    cur.load(rows, srow, x, norm_w, wave, K, block, lane);
+    cur.load(rows, srow, x, norm_w, wave, K, block, block_shift, lane);
   }
 
   // xs: raw x in LDS when NORM; part: GEMV_WAVES * R floats of LDS
@@ -245,7 +256,7 @@ struct stream_t {
     for (int b = 0; b < n_batches; ++b) {
       batch nxt;
       if (b + 1 < n_batches) {
-        nxt.load(rows, srow, x, norm_w, (b + 1) * GEMV_WAVES + wave, K, block, lane);
+        nxt.load(rows, srow, x, norm_w, (b + 1) * GEMV_WAVES + wave, K, block, block_shift, lane);
       }
       cur.fma(xs, rms_inv, b * GEMV_WAVES + wave, K, lane, a0, a1);
       cur = nxt;

@@ -9,6 +9,7 @@
 // and its one-launch-per-operation decode loop (a single new token runs the fused kernels).
 #include <assert.h>
 #include <stddef.h>
+#include <stdlib.h>
 #include <string.h>
 
 #include "model_impl.hpp"
@@ -473,7 +474,10 @@ short llama_context_impl::next_token(std::vector<short> const& new_tokens) {
     }
     decode_bound_ = bound;
     ++decode_calls_;
-    if (!decode_graph_ && decode_calls_ >= 2) {
+    // LLAMA_CU_NO_GRAPH=1 keeps every step eager: profilers that instrument graph launches have
+    // crashed on the host inside hipGraphLaunch on graphs of more than about 400 kernel nodes
+    static const bool no_graph = getenv("LLAMA_CU_NO_GRAPH") != nullptr && atoi(getenv("LLAMA_CU_NO_GRAPH")) != 0;
+    if (!decode_graph_ && decode_calls_ >= 2 && !no_graph) {
       LCU_CHECK(lcu_graph_begin_capture(stream_));
       enqueue_all();
       LCU_CHECK(lcu_graph_end_capture(stream_, &decode_graph_));

@@ -32,8 +32,9 @@ PKG = os.path.join(ROOT, "llama.cu_amd")
 HBM_PEAK_GBS = 8000.0      # MI355X HBM3E
 # HBM bytes per launch of the dominant kernel from rocprofv3 FETCH_SIZE / WRITE_SIZE, scaled by a
 # 256 MiB copy kernel read under the same counters (FETCH_SIZE reads half the bytes here): see
-# profiles/decode_ffn_up_kernel_llama7b_hbm_traffic.txt.  Counters are not read in this script.
-MEASURED_TRAFFIC = {"llama7b_fp16": 180639539}
+# profiles/decode_ffn_up_kernel_llama7b_hbm_traffic.txt and decode_u8_kernels_llama30b_counters.txt.
+# Counters are not read in this script.
+MEASURED_TRAFFIC = {"llama7b_fp16": 180641794, "llama30b_u8": 247164928}
 MFMA_F16_PEAK_TF = 2500.0  # dense fp16
 
 WORKLOADS = {

@@ -77,13 +77,25 @@ struct x_stage_t {
   }
 };
 
-// rms_norm applied to 8 elements in registers: fp16(w * fp16(x * rms_inv)), llama_cu.cu:103-106
+// rms_norm applied to 8 elements in registers: fp16(w * fp16(x * rms_inv)), llama_cu.cu:103-106.
+// x * rms_inv is rounded to fp32 and then to fp16 (two at a time, v_cvt_pk_f16_f32); the product
+// with the weight is one packed fp16 multiply: the fp32 product of two halves is exact, so
+// rounding it to fp16 is what the fp16 multiply itself does.  Three instructions per element
+// instead of seven: every workgroup of the logits GEMV normalises the whole row.
 __device__ __forceinline__ half8_t normed(half8_t x, half8_t w, float rms_inv) {
+  typedef float float2_t __attribute__((ext_vector_type(2)));
   half8_t r;
 #pragma unroll
-  for (int e = 0; e < 8; ++e) {
-    const half_t inner = round_f16((float)x[e] * rms_inv);
-    r[e] = round_f16((float)w[e] * (float)inner);
+  for (int e = 0; e < 8; e += 2) {
+    float2_t p;
+    p.x = (float)x[e] * rms_inv;
+    p.y = (float)x[e + 1] * rms_inv;
+    asm("" : "+v"(p));  // keeps the multiply and the conversion apart (see round_f16)
+    const half2_t inner = __builtin_convertvector(p, half2_t);
+    const half2_t ww = {w[e], w[e + 1]};
+    const half2_t res = ww * inner;
+    r[e] = res.x;
+    r[e + 1] = res.y;
   }
   return r;
 }
@@ -321,58 +333,74 @@ struct plain_tasks {
   }
 };
 
-// One of Wq / Wk / Wv (chosen per workgroup by the kernel): task = one interleaved pair (rows 2p,
-// 2p+1); RoPE on q and k (llama_cu.cu:381-387), results to q_out / the caches' row for this position
-template <bool U8>
+// One of Wq / Wk / Wv (chosen per workgroup by the kernel): a task is PAIRS interleaved pairs (rows
+// 2p, 2p+1) of that matrix; RoPE on q and k (llama_cu.cu:381-387), results to q_out / the caches'
+// row for this position
+template <bool U8, int PAIRS>
 struct qkv_tasks {
   const void* W;
   const half_t* S;
   half_t* dst;             // q_out, or the K / V cache row of this position
   const float2* rope_row;  // nullptr for V
   int dim, head_dim, nblk, first_task;
-  __device__ __forceinline__ void rows(int task, const uint8_t* (&rows)[2], const half_t* (&srow)[2]) const {
-    const int p = task - first_task;
+  __device__ __forceinline__ void rows(int task, const uint8_t* (&rows)[2 * PAIRS],
+                                       const half_t* (&srow)[2 * PAIRS]) const {
+    const int p0 = (task - first_task) * PAIRS;
 #pragma unroll
-    for (int r = 0; r < 2; ++r) {
-      rows[r] = row_ptr<U8>(W, 2 * p + r, dim);
-      srow[r] = U8 ? S + (size_t)(2 * p + r) * nblk : nullptr;
+    for (int r = 0; r < 2 * PAIRS; ++r) {
+      rows[r] = row_ptr<U8>(W, 2 * p0 + r, dim);
+      srow[r] = U8 ? S + (size_t)(2 * p0 + r) * nblk : nullptr;
     }
   }
-  __device__ __forceinline__ void finish(int task, const float (&acc)[2]) const {
-    const int p = task - first_task;
-    // the GEMV output is rounded to fp16 before RoPE reads it (llama_cu.cu:1144-1153)
-    const half_t h0 = round_f16(acc[0]), h1 = round_f16(acc[1]);
-    half2_t o;
-    if (rope_row == nullptr) {
-      o.x = h0;
-      o.y = h1;
-    } else {
-      const float2 cs = rope_row[((2 * p) % head_dim) / 2];
-      const float real = (float)h0, imag = (float)h1;
-      o.x = round_f16(fmaf(real, cs.x, -(imag * cs.y)));
-      o.y = round_f16(fmaf(real, cs.y, imag * cs.x));
+  __device__ __forceinline__ void finish(int task, const float (&acc)[2 * PAIRS]) const {
+#pragma unroll
+    for (int i = 0; i < PAIRS; ++i) {
+      const int p = (task - first_task) * PAIRS + i;
+      // the GEMV output is rounded to fp16 before RoPE reads it (llama_cu.cu:1144-1153)
+      const half_t h0 = round_f16(acc[2 * i]), h1 = round_f16(acc[2 * i + 1]);
+      half2_t o;
+      if (rope_row == nullptr) {
+        o.x = h0;
+        o.y = h1;
+      } else {
+        const float2 cs = rope_row[((2 * p) % head_dim) / 2];
+        const float real = (float)h0, imag = (float)h1;
+        o.x = round_f16(fmaf(real, cs.x, -(imag * cs.y)));
+        o.y = round_f16(fmaf(real, cs.y, imag * cs.x));
+      }
+      *reinterpret_cast<half2_t*>(dst + 2 * p) = o;
     }
-    *reinterpret_cast<half2_t*>(dst + 2 * p) = o;
   }
 };
 
-// W1 row j and W3 row j -> fp16 each -> fp16(silu(w1) * w3)  (llama_cu.cu:1180-1183, 533-539)
-template <bool U8>
+// PAIRS times: W1 row j and W3 row j -> fp16 each -> fp16(silu(w1) * w3)  (llama_cu.cu:1180-1183, 533-539)
+template <bool U8, int PAIRS>
 struct ffn_up_tasks {
   const void *w1, *w3;
   const half_t *s1, *s3;
   half_t* out;
-  int dim, nblk;
-  __device__ __forceinline__ void rows(int task, const uint8_t* (&rows)[2], const half_t* (&srow)[2]) const {
-    rows[0] = row_ptr<U8>(w1, task, dim);
-    rows[1] = row_ptr<U8>(w3, task, dim);
-    srow[0] = U8 ? s1 + (size_t)task * nblk : nullptr;
-    srow[1] = U8 ? s3 + (size_t)task * nblk : nullptr;
+  int dim, nblk, ffn;
+  __device__ __forceinline__ void rows(int task, const uint8_t* (&rows)[2 * PAIRS],
+                                       const half_t* (&srow)[2 * PAIRS]) const {
+#pragma unroll
+    for (int i = 0; i < PAIRS; ++i) {
+      const int j = min(task * PAIRS + i, ffn - 1);
+      rows[2 * i] = row_ptr<U8>(w1, j, dim);
+      rows[2 * i + 1] = row_ptr<U8>(w3, j, dim);
+      srow[2 * i] = U8 ? s1 + (size_t)j * nblk : nullptr;
+      srow[2 * i + 1] = U8 ? s3 + (size_t)j * nblk : nullptr;
+    }
   }
-  __device__ __forceinline__ void finish(int task, const float (&acc)[2]) const {
-    const float val = (float)round_f16(acc[0]);
-    const float gate = (float)round_f16(acc[1]);
-    out[task] = round_f16(val / (1.0f + exp_ieee(-val)) * gate);
+  __device__ __forceinline__ void finish(int task, const float (&acc)[2 * PAIRS]) const {
+#pragma unroll
+    for (int i = 0; i < PAIRS; ++i) {
+      const int j = task * PAIRS + i;
+      if (j < ffn) {
+        const float val = (float)round_f16(acc[2 * i]);
+        const float gate = (float)round_f16(acc[2 * i + 1]);
+        out[j] = round_f16(val / (1.0f + exp_ieee(-val)) * gate);
+      }
+    }
   }
 };
 
@@ -404,7 +432,7 @@ __global__ __launch_bounds__(GEMV_THREADS) void gemv_kernel(half_t* __restrict__
   st.run(xs, rms_inv, part);
 }
 
-template <bool U8, int U, int XN>
+template <bool U8, int U, int XN, int PAIRS>
 __global__ __launch_bounds__(GEMV_THREADS) void decode_qkv_kernel(
     half_t* __restrict__ q_out, half_t* __restrict__ k_row, half_t* __restrict__ v_row, const half_t* __restrict__ x,
     const half_t* __restrict__ norm_w, const void* __restrict__ wq, const void* __restrict__ wk,
@@ -413,7 +441,7 @@ __global__ __launch_bounds__(GEMV_THREADS) void decode_qkv_kernel(
     const int* __restrict__ pos_dev, int max_pos) {
   extern __shared__ half_t xs[];
   __shared__ float red[8];
-  __shared__ float part[GEMV_WAVES * 2];
+  __shared__ float part[GEMV_WAVES * 2 * PAIRS];
   if (pos_dev) {  // position kept on the device (graph replay): the row pointers arrive as bases
     const int pos = min(max(*pos_dev, 0), max_pos);
     k_row += (size_t)pos * dim;
@@ -422,14 +450,15 @@ __global__ __launch_bounds__(GEMV_THREADS) void decode_qkv_kernel(
   }
   // one task per workgroup, so the matrix is chosen here, once, from the kernel arguments (a
   // per-task choice inside the task struct made the compiler index the struct in scratch memory)
-  const int half_dim = dim / 2;
-  const int which = blockIdx.x / half_dim;
+  const int tasks_per_matrix = dim / 2 / PAIRS;
+  const int which = blockIdx.x / tasks_per_matrix;
   const void* W = which == 0 ? wq : (which == 1 ? wk : wv);
   const half_t* S = which == 0 ? sq : (which == 1 ? sk : sv);
   half_t* dst = which == 0 ? q_out : (which == 1 ? k_row : v_row);
-  qkv_tasks<U8> tk{W, S, dst, which == 2 ? nullptr : rope_row, dim, head_dim, U8 ? dim / block : 0, which * half_dim};
+  qkv_tasks<U8, PAIRS> tk{W, S, dst, which == 2 ? nullptr : rope_row, dim, head_dim, U8 ? dim / block : 0,
+                          which * tasks_per_matrix};
   constexpr bool NORM = XN > 0;
-  stream_t<U8, 2, U, NORM, qkv_tasks<U8>> st(tk, x, norm_w, dim, block, blockIdx.x);
+  stream_t<U8, 2 * PAIRS, U, NORM, qkv_tasks<U8, PAIRS>> st(tk, x, norm_w, dim, block, blockIdx.x);
   float rms_inv = 1.0f;
   if constexpr (NORM) {
     x_stage_t<XN> xp;
@@ -444,17 +473,17 @@ __global__ __launch_bounds__(GEMV_THREADS) void decode_qkv_kernel(
   st.run(xs, rms_inv, part);
 }
 
-template <bool U8, int U, int XN>
+template <bool U8, int U, int XN, int PAIRS>
 __global__ __launch_bounds__(GEMV_THREADS) void decode_ffn_up_kernel(
     half_t* __restrict__ out, const half_t* __restrict__ x, const half_t* __restrict__ norm_w,
     const void* __restrict__ w1, const void* __restrict__ w3, const half_t* __restrict__ s1,
     const half_t* __restrict__ s3, int block, int dim, int ffn, float eps) {
   extern __shared__ half_t xs[];
   __shared__ float red[8];
-  __shared__ float part[GEMV_WAVES * 2];
-  ffn_up_tasks<U8> tk{w1, w3, s1, s3, out, dim, U8 ? dim / block : 0};
+  __shared__ float part[GEMV_WAVES * 2 * PAIRS];
+  ffn_up_tasks<U8, PAIRS> tk{w1, w3, s1, s3, out, dim, U8 ? dim / block : 0, ffn};
   constexpr bool NORM = XN > 0;
-  stream_t<U8, 2, U, NORM, ffn_up_tasks<U8>> st(tk, x, norm_w, dim, block, blockIdx.x);
+  stream_t<U8, 2 * PAIRS, U, NORM, ffn_up_tasks<U8, PAIRS>> st(tk, x, norm_w, dim, block, blockIdx.x);
   float rms_inv = 1.0f;
   if constexpr (NORM) {
     x_stage_t<XN> xp;
@@ -505,7 +534,10 @@ int gemv_f16(half_t* out, const half_t* x, const half_t* W, int K, int N, float 
 
 int gemv_u8(half_t* out, const half_t* x, const uint8_t* W, const half_t* S, int K, int N, int block, float beta,
             hipStream_t st) {
-  if (N >= 8192) {
+  // four rows per workgroup where that still gives most compute units eight workgroups: x (as many
+  // bytes as two rows of codes) is then fetched half as often (30B shapes: W1/W3 41.5 -> 38.9 us,
+  // the logits 216 MB in 34 us); at N = 4096 it would leave half the workgroup slots empty
+  if (N >= 6144) {
     gemv_kernel<true, 4, 1, 0><<<(N + 3) / 4, GEMV_THREADS, 0, st>>>(out, x, nullptr, W, S, K, N, block, beta, 0.f);
   } else {
     gemv_kernel<true, 2, 1, 0><<<(N + 1) / 2, GEMV_THREADS, 0, st>>>(out, x, nullptr, W, S, K, N, block, beta, 0.f);
@@ -546,13 +578,13 @@ int lcu_decode_qkv(void* q_out_dev, void* k_cache_dev, void* v_cache_dev, const 
     LCU_REQUIRE(sk_dev && sv_dev, "lcu_decode_qkv: quantised weights need scales");
     if (norm_w_dev) {
       with_x_pieces(dim, [&](auto xn) {
-        decode_qkv_kernel<true, 1, decltype(xn)::value><<<grid, GEMV_THREADS, decltype(xn)::value * 4096, st>>>(
+        decode_qkv_kernel<true, 1, decltype(xn)::value, 1><<<grid, GEMV_THREADS, decltype(xn)::value * 4096, st>>>(
             (half_t*)q_out_dev, k_row, v_row, (const half_t*)x_dev, (const half_t*)norm_w_dev, wq_dev, wk_dev, wv_dev,
             (const half_t*)sq_dev, (const half_t*)sk_dev, (const half_t*)sv_dev, block, dim, head_dim, eps, rope_row,
             (const int*)pos_dev, table_positions - 1);
       });
     } else {
-      decode_qkv_kernel<true, 1, 0><<<grid, GEMV_THREADS, 0, st>>>(
+      decode_qkv_kernel<true, 1, 0, 2><<<grid / 2, GEMV_THREADS, 0, st>>>(
           (half_t*)q_out_dev, k_row, v_row, (const half_t*)x_dev, nullptr, wq_dev, wk_dev, wv_dev,
           (const half_t*)sq_dev, (const half_t*)sk_dev, (const half_t*)sv_dev, block, dim, head_dim, eps, rope_row, (const int*)pos_dev,
           table_positions - 1);
@@ -560,12 +592,12 @@ int lcu_decode_qkv(void* q_out_dev, void* k_cache_dev, void* v_cache_dev, const 
   } else {
     if (norm_w_dev) {
       with_x_pieces(dim, [&](auto xn) {
-        decode_qkv_kernel<false, 2, decltype(xn)::value><<<grid, GEMV_THREADS, decltype(xn)::value * 4096, st>>>(
+        decode_qkv_kernel<false, 2, decltype(xn)::value, 1><<<grid, GEMV_THREADS, decltype(xn)::value * 4096, st>>>(
             (half_t*)q_out_dev, k_row, v_row, (const half_t*)x_dev, (const half_t*)norm_w_dev, wq_dev, wk_dev, wv_dev,
             nullptr, nullptr, nullptr, 0, dim, head_dim, eps, rope_row, (const int*)pos_dev, table_positions - 1);
       });
     } else {
-      decode_qkv_kernel<false, 2, 0><<<grid, GEMV_THREADS, 0, st>>>(
+      decode_qkv_kernel<false, 2, 0, 1><<<grid, GEMV_THREADS, 0, st>>>(
           (half_t*)q_out_dev, k_row, v_row, (const half_t*)x_dev, nullptr, wq_dev, wk_dev, wv_dev, nullptr, nullptr,
           nullptr, 0, dim, head_dim, eps, rope_row, (const int*)pos_dev, table_positions - 1);
     }
@@ -588,24 +620,24 @@ int lcu_decode_ffn_up(void* out_dev, const void* x_dev, const void* norm_w_dev, 
     LCU_REQUIRE(s3_dev != nullptr, "lcu_decode_ffn_up: quantised weights need scales");
     if (norm_w_dev) {
       with_x_pieces(dim, [&](auto xn) {
-        decode_ffn_up_kernel<true, 1, decltype(xn)::value><<<grid, GEMV_THREADS, decltype(xn)::value * 4096, st>>>(
+        decode_ffn_up_kernel<true, 1, decltype(xn)::value, 1><<<grid, GEMV_THREADS, decltype(xn)::value * 4096, st>>>(
             (half_t*)out_dev, (const half_t*)x_dev, (const half_t*)norm_w_dev, w1_dev, w3_dev, (const half_t*)s1_dev,
             (const half_t*)s3_dev, block, dim, ffn, eps);
       });
     } else {
-      decode_ffn_up_kernel<true, 1, 0><<<grid, GEMV_THREADS, 0, st>>>(
+      decode_ffn_up_kernel<true, 1, 0, 2><<<(grid + 1) / 2, GEMV_THREADS, 0, st>>>(
           (half_t*)out_dev, (const half_t*)x_dev, nullptr, w1_dev, w3_dev, (const half_t*)s1_dev,
           (const half_t*)s3_dev, block, dim, ffn, eps);
     }
   } else {
     if (norm_w_dev) {
       with_x_pieces(dim, [&](auto xn) {
-        decode_ffn_up_kernel<false, 2, decltype(xn)::value><<<grid, GEMV_THREADS, decltype(xn)::value * 4096, st>>>(
+        decode_ffn_up_kernel<false, 2, decltype(xn)::value, 1><<<grid, GEMV_THREADS, decltype(xn)::value * 4096, st>>>(
             (half_t*)out_dev, (const half_t*)x_dev, (const half_t*)norm_w_dev, w1_dev, w3_dev, nullptr, nullptr, 0, dim,
             ffn, eps);
       });
     } else {
-      decode_ffn_up_kernel<false, 2, 0><<<grid, GEMV_THREADS, 0, st>>>(
+      decode_ffn_up_kernel<false, 2, 0, 1><<<grid, GEMV_THREADS, 0, st>>>(
           (half_t*)out_dev, (const half_t*)x_dev, nullptr, w1_dev, w3_dev, nullptr, nullptr, 0, dim, ffn, eps);
     }
   }

@@ -374,9 +374,17 @@ void llama_context_impl::enqueue_head(int n) {
   const int dim = p.dim, vocab = p.n_vocab;
   const int block = p.q_type == quantization_type::uint8 ? p.quantization_block_size : 0;
   char* x = (char*)t_embed_.data();
-  LCU_CHECK(lcu_decode_logits(t_logits_.data(), x + (size_t)(n - 1) * dim * 2, model_->norm.data(),
-                              model_->output.data.data(), model_->output.scales.data(), block, dim, vocab, p.norm_eps,
-                              stream_));
+  if (block > 0) {
+    // uint8 weights: the GEMV is bound by its vector instructions, and normalising the row in each of
+    // its 16 000 workgroups costs more there (60 us) than a norm launch of its own (6 + 39 us)
+    LCU_CHECK(lcu_rmsnorm(t_norm_.data(), x + (size_t)(n - 1) * dim * 2, model_->norm.data(), 1, dim, p.norm_eps, stream_));
+    LCU_CHECK(lcu_gemm_f16u8_nt(t_logits_.data(), t_norm_.data(), model_->output.data.data(),
+                                model_->output.scales.data(), 1, dim, vocab, block, 0.0f, stream_));
+  } else {
+    LCU_CHECK(lcu_decode_logits(t_logits_.data(), x + (size_t)(n - 1) * dim * 2, model_->norm.data(),
+                                model_->output.data.data(), model_->output.scales.data(), block, dim, vocab, p.norm_eps,
+                                stream_));
+  }
   // the first maximum of the fp16 probabilities is found on the device; 4 bytes go back to the host
   LCU_CHECK(lcu_softmax_argmax(t_probs_.data(), t_argmax_.data(), t_logits_.data(), vocab, temperature_, stream_));
   if (sampling_) {  // 1202-1203; the random bits of this step are in t_step_

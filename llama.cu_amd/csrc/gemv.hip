@@ -18,8 +18,10 @@
 //     LDS, thread 0 applies the epilogue (residual add, RoPE, SiLU*mul) and rounds once to fp16
 // uint8 weights are dequantised in packed fp16 to bit-for-bit fp16((q - 127.5) * scale), the value
 // the reference feeds its tensor cores (287-289, 336-341): see dequant2_fma / dequant2.  The
-// products then go through v_dot2_f32_f16 (two multiply-adds per instruction, fp32 accumulate):
-// the dequantisation arithmetic, not HBM, is what bounds this kernel on large matrices.
+// products then go through v_dot2_f32_f16 (two multiply-adds per instruction, fp32 accumulate;
+// the instruction aligns and cuts its three addends in a way of its own, which the oracle's
+// kernel-order flavour restates from measured samples): the dequantisation arithmetic, not HBM,
+// is what bounds this kernel on large matrices.
 #include "common.hpp"
 
 #include <type_traits>

@@ -58,8 +58,9 @@ void orc_dequantize_absmax_u8(uint16_t* out, const uint16_t* scales, const uint8
  *            context created with it also takes the attention and the logits softmax of a
  *            one-token call in the order of the HIP kernels.  Any fp32 order is as good a restatement
  *            of the reference's tensor-core sums as another (their order is the hardware's); this
- *            one lets a decode step be compared with the GPU bit for bit (fp16 weights) instead
- *            of within a tolerance.  Pinned by the same float64 / identity / one-hot checks as the
+ *            one lets a decode step be compared with the GPU bit for bit (fp16 and uint8 weights;
+ *            the uint8 kernels pair their products through v_dot2_f32_f16, restated from
+ *            measured samples: dot2_f32_f16 in oracle.cpp) instead of within a tolerance.  Pinned by the same float64 / identity / one-hot checks as the
  *            other flavours (tests/test_oracle_ops.py). */
 void orc_matmul_nt(uint16_t* out, const uint16_t* lhs, const uint16_t* rhs, int M, int K, int N,
                    float beta, int flavour);
@@ -112,6 +113,10 @@ void orc_error_stats(float* out3, const uint16_t* a, const uint16_t* b, size_t n
 /* e^x as every softmax and SiLU of this oracle takes it: IEEE operations only (the reference calls
  * CUDA's expf, llama_cu.cu:463, 497, 537); pinned against float64 exp to one ulp. */
 void orc_exp_f32(float* out, const float* in, size_t n);
+
+/* out[i] = v_dot2_f32_f16(a[2i..2i+1], b[2i..2i+1], c[i]) as gfx950 computes it (a, b: fp16 bit
+ * patterns); restated from measured samples, see dot2_f32_f16 in oracle.cpp. */
+void orc_dot2_f32_f16(float* out, const uint16_t* a, const uint16_t* b, const float* c, size_t n);
 /* Attention of one new token (q [dim], the first T rows of k (rotated) and v [T][dim], head_dim 128)
  * and softmax with temperature over one row of n logits (n a multiple of 8 up to 32768): the
  * arithmetic of llama_cu.cu:400-428, 433-499, 511-531 with the sums taken in the order of this

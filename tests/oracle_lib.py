@@ -41,6 +41,8 @@ def lib():
         L.orc_silu_mul.argtypes = [vp, vp, vp, sz]
         L.orc_exp_f32.argtypes = [vp, vp, sz]
         L.orc_exp_f32.restype = None
+        L.orc_dot2_f32_f16.argtypes = [vp, vp, vp, vp, sz]
+        L.orc_dot2_f32_f16.restype = None
         L.orc_attention_decode_kernel_order.argtypes = [vp, vp, vp, vp, i, i, i]
         L.orc_attention_decode_kernel_order.restype = None
         L.orc_softmax_logits_kernel_order.argtypes = [vp, vp, i, f]
@@ -176,6 +178,17 @@ def matmul_qkv(p, v, n_heads):
 def attention(q, k, v, n_heads, start_pos):
     """matmul_qk -> softmax_rows -> matmul_qkv, llama_cu.cu:1161-1171."""
     return matmul_qkv(softmax_rows(matmul_qk(q, k, n_heads, start_pos)), v, n_heads)
+
+
+def dot2_f32_f16(a, b, c):
+    """a, b: (n, 2) fp16 bit patterns (uint16), c: (n,) float32 -> what v_dot2_f32_f16 returns"""
+    a = np.ascontiguousarray(a, dtype=np.uint16)
+    b = np.ascontiguousarray(b, dtype=np.uint16)
+    c = np.ascontiguousarray(c, dtype=np.float32)
+    assert a.shape == b.shape == (c.size, 2)
+    out = np.empty_like(c)
+    lib().orc_dot2_f32_f16(_p(out), _p(a), _p(b), _p(c), c.size)
+    return out
 
 
 def exp_f32(x):

@@ -1,4 +1,4 @@
-// Measures v_dot2_f32_f16 on the GPU: 2^21 seeded (a, b, c) samples and what the instruction
+// Measures v_dot2_f32_f16 on the GPU: 3 * 2^20 seeded (a, b, c) samples and what the instruction
 // returns for them, written as raw arrays (a: 2 fp16 per sample, b: 2 fp16, c: fp32, out: fp32).
 // make_dot2_fixture.py picks the samples kept in dot2_gfx950.npz.
 //   hipcc --offload-arch=gfx950 -O2 -o dot2_probe tests/golden/dot2_probe.hip && ./dot2_probe dot2.bin
@@ -29,7 +29,7 @@ int main(int argc, char** argv) {
     printf("usage: %s <output file>\n", argv[0]);
     return 2;
   }
-  const int n = 1 << 21, n_first = 1 << 20;
+  const int n = 3 << 20, n_first = 1 << 20, n_second = 2 << 20;
   std::vector<float> hc(n), ho(n);
   std::vector<_Float16> fa(2 * n), fb(2 * n);
   std::mt19937_64 rng(1);
@@ -48,7 +48,7 @@ int main(int argc, char** argv) {
   }
   // second half: halves drawn by bit pattern (exponent field 0..20, so one in 21 is subnormal), c
   // placed -6..+14 binades from the larger product with a random 24-bit mantissa
-  for (int i = n_first; i < n; ++i) {
+  for (int i = n_first; i < n_second; ++i) {
     uint16_t h[4];
     for (int j = 0; j < 4; ++j) {
       const uint64_t r = rng();
@@ -63,6 +63,24 @@ int main(int argc, char** argv) {
     const float mant = 1.0f + (float)(r & 0x7fffff) * 0x1p-23f;
     hc[i] = big == 0.f ? mant : ldexpf(mant, ilogbf(big) + gap);
     if ((r >> 60) & 1) hc[i] = -hc[i];
+  }
+  // third part: c so close to a power of two, 6..13 binades above the products, that the products
+  // carry the sum across it (the result's exponent is then not that of the largest addend)
+  for (int i = n_second; i < n; ++i) {
+    uint16_t h[4];
+    for (int j = 0; j < 4; ++j) {
+      const uint64_t r = rng();
+      h[j] = (uint16_t)(((r >> 40) & 1) << 15 | (8 + (r >> 20) % 13) << 10 | (r & 0x3ff));
+    }
+    memcpy(&fa[2 * i], &h[0], 4);
+    memcpy(&fb[2 * i], &h[2], 4);
+    const double p0 = (double)fa[2 * i] * (double)fb[2 * i], p1 = (double)fa[2 * i + 1] * (double)fb[2 * i + 1];
+    const double sum = p0 + p1, big = fabs(p0) > fabs(p1) ? fabs(p0) : fabs(p1);
+    const uint64_t r = rng();
+    const double edge = ldexp(1.0, ilogb(big) + 6 + (int)((r >> 32) % 8));
+    const double u = (double)(r & 0xffffff) * 0x1p-24, sign = (r >> 60) & 1 ? -1.0 : 1.0;
+    // products against c: c just beyond the edge, the sum just inside it; with c: the other way round
+    hc[i] = (float)(sign * sum < 0 ? sign * (edge + u * fabs(sum)) : sign * (edge - u * fabs(sum)));
   }
   half2_t *da, *db;
   float *dc, *dout;

@@ -188,9 +188,12 @@ def test_gemm_f16(gpu, M, K, N):
     ref = O.matmul_nt(x, w)
     assert G.max_abs_rel(got, ref) <= TOL
     assert G.ulp_mismatch(got, ref) < 0.05
+    # the kernel-order flavour restates the matrix cores' sums and the dispatcher's cut of K: bit for bit
+    assert G.ulp_mismatch(got, O.matmul_nt(x, w, flavour=2)) == 0.0, O.gemm_plan(M, K, N)
     old = normal((M, N), 0, 302, 1.0)
     got = G.gemm_f16(x, w, beta=1.0, out=old)
     assert G.max_abs_rel(got, O.matmul_nt(x, w, beta=1.0, out=old)) <= TOL
+    assert G.ulp_mismatch(got, O.matmul_nt(x, w, beta=1.0, out=old, flavour=2)) == 0.0
     G.release()
 
 
@@ -222,6 +225,7 @@ def test_gemm_u8(gpu, M, K, N):
     ref = O.matmul_nt_u8(x, codes, scales, 128)
     assert G.max_abs_rel(got, ref) <= TOL
     assert G.ulp_mismatch(got, ref) < 0.05
+    assert G.ulp_mismatch(got, O.matmul_nt_u8(x, codes, scales, 128, flavour=2)) == 0.0, O.gemm_plan(M, K, N, True)
     # row r of the M-row product equals the single-row product (decode path) within tolerance
     one = G.gemm_u8(x[3:4], codes, scales, 128)
     assert G.max_abs_rel(one, got[3:4]) <= TOL
@@ -251,6 +255,8 @@ def test_gemm_multi_matches_separate_calls(gpu, M, K, N, count):
         got = G.host(outs[g], (M, N))
         assert G.max_abs_rel(got, sep[g]) <= TOL and G.ulp_mismatch(got, sep[g]) < 0.05, g
         assert G.max_abs_rel(got, O.matmul_nt(x, ws[g])) <= TOL, g
+        if K % 8 == 0:
+            assert G.ulp_mismatch(got, O.matmul_nt_kernel_order(x, ws[g], n_mats=count)) == 0.0, g
     if K % 128 == 0:
         q = [O.quantize_absmax_u8(w, 128) for w in ws]
         cd = [G.dev_keep(c) for c, _ in q]
@@ -263,6 +269,8 @@ def test_gemm_multi_matches_separate_calls(gpu, M, K, N, count):
             got = G.host(outs[g], (M, N))
             assert G.max_abs_rel(got, sep[g]) <= TOL and G.ulp_mismatch(got, sep[g]) < 0.05, g
             assert G.max_abs_rel(got, O.matmul_nt_u8(x, q[g][0], q[g][1], 128)) <= TOL, g
+            assert G.ulp_mismatch(got, O.matmul_nt_kernel_order(x, codes=q[g][0], scales=q[g][1], block=128,
+                                                               n_mats=count)) == 0.0, g
     # beta = 1: every output starts from its own earlier contents
     olds = [normal((M, N), 0, 1650 + g, 1.0) for g in range(count)]
     for g in range(count):

@@ -1116,8 +1116,16 @@ static void rope_rows(const orc_context* c, uint16_t* out, const uint16_t* in, i
   }
 }
 
-static void mm(const orc_context* c, uint16_t* out, const uint16_t* lhs, const orc_tensor& w, int M, float beta) {
+// n_mats: how many products of this shape the HIP host code launches together (flavour 2 only: it
+// decides how the kernels cut K)
+static void mm(const orc_context* c, uint16_t* out, const uint16_t* lhs, const orc_tensor& w, int M, float beta,
+               int n_mats = 1) {
   // llama_cu.cu:1498-1523
+  if (c->flavour == 2 && M > 1 && w.cols % (w.quantised ? 16 : 8) == 0) {
+    orc_matmul_nt_kernel_order(out, lhs, w.quantised ? nullptr : w.h.data(), w.quantised ? w.q.data() : nullptr,
+                               w.quantised ? w.h.data() : nullptr, M, w.cols, w.rows, c->model->qblock, beta, n_mats);
+    return;
+  }
   if (w.quantised) {
     orc_matmul_nt_u8(out, lhs, w.q.data(), w.h.data(), M, w.cols, w.rows, c->model->qblock, beta, c->flavour);
   } else {
@@ -1231,6 +1239,120 @@ static void attention_decode_kernel_order(uint16_t* out, const uint16_t* q, cons
   }
 }
 
+// csrc/attention.hip, several new rows (prefill_attention_kernel): per head, a tile of BR rows sees the
+// cache columns 0 .. Tc - 1, Tc = its last row's causal span rounded up to 64 (masked columns hold
+// -inf).  A score is a chain of 16 matrix-core steps of eight over the 128 head dimensions from 0,
+// divided by sqrt(128) and rounded to fp16.  Softmax of a row by one wavefront: lane l takes the
+// column pairs l, l + 64, ...; the maximum; per lane the sum of (exp(x0 - m) + exp(x1 - m)) over its
+// pairs in order, the 64 lane sums added pairwise between neighbours; p = fp16(exp(x - m) / sum).
+// An output element is a chain of Tc / 8 steps of eight over ascending cache rows from 0, rounded
+// to fp16.  head_dim must be 128.
+static void attention_prefill_kernel_order(uint16_t* out, const uint16_t* q, const uint16_t* k, const uint16_t* v,
+                                           int n_new, int T, int start_pos, int dim, int n_heads) {
+  const float denom = sqrtf(128.0f);
+  const long wgs32 = (long)((n_new + 31) / 32) * n_heads;
+  const int BR = (wgs32 < 1024 && T <= 1024) ? 16 : 32;
+  const int Tc_max = (T + 63) / 64 * 64;
+#pragma omp parallel
+  {
+    std::vector<double> kT((size_t)128 * Tc_max), skT((size_t)128 * Tc_max);  // [d][col]
+    std::vector<double> vd((size_t)Tc_max * 128), svd((size_t)Tc_max * 128);  // [row][d]
+    std::vector<double> pd(Tc_max), spd(Tc_max);
+    std::vector<uint16_t> sc(Tc_max);
+#pragma omp for schedule(dynamic, 1)
+    for (int h = 0; h < n_heads; ++h) {
+      for (int c = 0; c < Tc_max; ++c) {
+        const int src = c < T ? c : T - 1;  // rows past T are read but meet p = 0 only
+        for (int d = 0; d < 128; d += 4) {
+          float f[4];
+          for (int i = 0; i < 4; ++i) f[i] = h2f(k[(size_t)src * dim + h * 128 + d + i]);
+          const __m256d kv = _mm256_cvtps_pd(_mm_loadu_ps(f));
+          double tmp[4], stmp[4];
+          _mm256_storeu_pd(tmp, kv);
+          _mm256_storeu_pd(stmp, half_scale_or_zero(kv));
+          for (int i = 0; i < 4; ++i) {
+            kT[(size_t)(d + i) * Tc_max + c] = tmp[i];
+            skT[(size_t)(d + i) * Tc_max + c] = stmp[i];
+          }
+          for (int i = 0; i < 4; ++i) f[i] = h2f(v[(size_t)src * dim + h * 128 + d + i]);
+          const __m256d vv = _mm256_cvtps_pd(_mm_loadu_ps(f));
+          _mm256_storeu_pd(&vd[(size_t)c * 128 + d], vv);
+          _mm256_storeu_pd(&svd[(size_t)c * 128 + d], half_scale_or_zero(vv));
+        }
+      }
+      for (int r = 0; r < n_new; ++r) {
+        const int r0 = r / BR * BR;
+        const int last_row = std::min(r0 + BR, n_new) - 1;
+        const int c_end = std::min(T, last_row + start_pos + 1);
+        const int Tc = (c_end + 63) / 64 * 64;
+        const int visible = std::min(T, r + start_pos + 1);  // columns 0 .. visible - 1 are not masked
+        double qd[128], sqd[128];
+        for (int d = 0; d < 128; d += 4) {
+          float f[4];
+          for (int i = 0; i < 4; ++i) f[i] = h2f(q[(size_t)r * dim + h * 128 + d + i]);
+          const __m256d qv = _mm256_cvtps_pd(_mm_loadu_ps(f));
+          _mm256_storeu_pd(qd + d, qv);
+          _mm256_storeu_pd(sqd + d, half_scale_or_zero(qv));
+        }
+        for (int c = 0; c < Tc; c += 4) {
+          if (c >= visible) {
+            for (int i = 0; i < 4; ++i) sc[c + i] = 0xfc00;  // -inf
+            continue;
+          }
+          __m256d acc = _mm256_setzero_pd();
+          for (int d = 0; d < 128; d += 8) {
+            __m256d a[8], sa[8], b[8], sb[8];
+            for (int i = 0; i < 8; ++i) {
+              a[i] = _mm256_broadcast_sd(qd + d + i);
+              sa[i] = _mm256_broadcast_sd(sqd + d + i);
+              b[i] = _mm256_loadu_pd(&kT[(size_t)(d + i) * Tc_max + c]);
+              sb[i] = _mm256_loadu_pd(&skT[(size_t)(d + i) * Tc_max + c]);
+            }
+            acc = mfma_step8(acc, a, sa, b, sb);
+          }
+          float res[4];
+          _mm_storeu_ps(res, _mm256_cvtpd_ps(acc));
+          for (int i = 0; i < 4; ++i) sc[c + i] = c + i < visible ? f2h(res[i] / denom) : 0xfc00;
+        }
+        float m = -INFINITY;
+        for (int c = 0; c < Tc; ++c) m = fmaxf(m, h2f(sc[c]));
+        float lanes[64];
+        for (int l = 0; l < 64; ++l) {
+          float sum = 0.0f;
+          for (int i = l; i < Tc / 2; i += 64) {
+            sum += exp_ieee(h2f(sc[2 * i]) - m) + exp_ieee(h2f(sc[2 * i + 1]) - m);
+          }
+          lanes[l] = sum;
+        }
+        const float total = tree64(lanes);
+        for (int c = 0; c < Tc; c += 4) {
+          float f[4];
+          for (int i = 0; i < 4; ++i) f[i] = h2f(f2h(exp_ieee(h2f(sc[c + i]) - m) / total));
+          const __m256d pv = _mm256_cvtps_pd(_mm_loadu_ps(f));
+          _mm256_storeu_pd(&pd[c], pv);
+          _mm256_storeu_pd(&spd[c], half_scale_or_zero(pv));
+        }
+        for (int d = 0; d < 128; d += 4) {
+          __m256d acc = _mm256_setzero_pd();
+          for (int c = 0; c < Tc; c += 8) {
+            __m256d a[8], sa[8], b[8], sb[8];
+            for (int i = 0; i < 8; ++i) {
+              a[i] = _mm256_broadcast_sd(&pd[c + i]);
+              sa[i] = _mm256_broadcast_sd(&spd[c + i]);
+              b[i] = _mm256_loadu_pd(&vd[(size_t)(c + i) * 128 + d]);
+              sb[i] = _mm256_loadu_pd(&svd[(size_t)(c + i) * 128 + d]);
+            }
+            acc = mfma_step8(acc, a, sa, b, sb);
+          }
+          float res[4];
+          _mm_storeu_ps(res, _mm256_cvtpd_ps(acc));
+          for (int i = 0; i < 4; ++i) out[(size_t)r * dim + h * 128 + d + i] = f2h(res[i]);
+        }
+      }
+    }
+  }
+}
+
 // softmax_argmax_kernel of csrc/elementwise.hip (n a multiple of 8, at most 32768): thread t of 1024
 // owns the 8-element pieces t, t + 1024, ... and adds their exponentials in ascending order; the 64
 // lanes of a wavefront are summed pairwise between neighbours; the 16 wavefront sums are added in
@@ -1285,6 +1407,11 @@ void orc_attention_decode_kernel_order(uint16_t* out, const uint16_t* q, const u
   attention_decode_kernel_order(out, q, k, v, T, dim, n_heads);
 }
 
+void orc_attention_prefill_kernel_order(uint16_t* out, const uint16_t* q, const uint16_t* k, const uint16_t* v, int n_new,
+                                        int T, int start_pos, int dim, int n_heads) {
+  attention_prefill_kernel_order(out, q, k, v, n_new, T, start_pos, dim, n_heads);
+}
+
 void orc_softmax_logits_kernel_order(uint16_t* out, const uint16_t* in, int n, float temp) {
   softmax_logits_kernel_order(out, in, n, temp);
 }
@@ -1309,9 +1436,9 @@ int orc_context_next_token(orc_context* c, const int16_t* tokens, int n, uint16_
     uint16_t* kc = c->k[l].data();
     uint16_t* vc = c->v[l].data();
     orc_rms_norm(norm.data(), x.data(), L.attn_norm.data(), n, dim, m->norm_eps);  // 1129
-    mm(c, xq.data(), norm.data(), L.wq, n, 0.0f);                                  // 1144
+    mm(c, xq.data(), norm.data(), L.wq, n, 0.0f, 3);                               // 1144
     rope_rows(c, xq.data(), xq.data(), n, sp);                                     // 1146
-    mm(c, kc + (size_t)sp * dim, norm.data(), L.wk, n, 0.0f);                      // 1150
+    mm(c, kc + (size_t)sp * dim, norm.data(), L.wk, n, 0.0f, 3);                   // 1150
     const uint16_t* krot;
     if (c->literal_rope) {
       rope_rows(c, xk.data(), kc, T, 0);                                           // 1152
@@ -1320,9 +1447,11 @@ int orc_context_next_token(orc_context* c, const int16_t* tokens, int n, uint16_
       rope_rows(c, kc + (size_t)sp * dim, kc + (size_t)sp * dim, n, sp);
       krot = kc;
     }
-    mm(c, vc + (size_t)sp * dim, norm.data(), L.wv, n, 0.0f);                      // 1156
+    mm(c, vc + (size_t)sp * dim, norm.data(), L.wv, n, 0.0f, 3);                   // 1156
     if (c->flavour == 2 && n == 1 && dim == H * 128) {
       attention_decode_kernel_order(att.data(), xq.data(), krot, vc, T, dim, H);   // 1163-1170
+    } else if (c->flavour == 2 && dim == H * 128) {
+      attention_prefill_kernel_order(att.data(), xq.data(), krot, vc, n, T, sp, dim, H);
     } else {
       orc_matmul_qk(qk.data(), xq.data(), krot, n, T, dim, H, sp);                 // 1163
       orc_softmax_rows(qk.data(), qk.data(), H * n, T, 1.0f);                      // 1166
@@ -1330,8 +1459,8 @@ int orc_context_next_token(orc_context* c, const int16_t* tokens, int n, uint16_
     }
     mm(c, x.data(), att.data(), L.wo, n, 1.0f);                                    // 1174
     orc_rms_norm(norm.data(), x.data(), L.ffn_norm.data(), n, dim, m->norm_eps);   // 1176
-    mm(c, w1.data(), norm.data(), L.w1, n, 0.0f);                                  // 1180
-    mm(c, w3.data(), norm.data(), L.w3, n, 0.0f);                                  // 1181
+    mm(c, w1.data(), norm.data(), L.w1, n, 0.0f, 2);                               // 1180
+    mm(c, w3.data(), norm.data(), L.w3, n, 0.0f, 2);                               // 1181
     orc_silu_mul(silu.data(), w1.data(), w3.data(), (size_t)n * ffn);              // 1183
     mm(c, x.data(), silu.data(), L.w2, n, 1.0f);                                   // 1185
   }

@@ -139,6 +139,11 @@ void orc_dot2_f32_f16(float* out, const uint16_t* a, const uint16_t* b, const fl
  * against orc_matmul_qk / orc_softmax_rows / orc_matmul_qkv within fp32 summation accuracy. */
 void orc_attention_decode_kernel_order(uint16_t* out, const uint16_t* q, const uint16_t* k, const uint16_t* v, int T,
                                        int dim, int n_heads);
+/* lcu_attention with n_new > 1 in the order of csrc/attention.hip (head_dim 128): scores and
+ * weighted sums as chains of matrix-core steps, the row softmax summed as its wavefront sums it. */
+void orc_attention_prefill_kernel_order(uint16_t* out, const uint16_t* q, const uint16_t* k, const uint16_t* v, int n_new,
+                                        int T, int start_pos, int dim, int n_heads);
+
 void orc_softmax_logits_kernel_order(uint16_t* out, const uint16_t* in, int n, float temp);
 
 /* ---- whole model: llama_cu.cu:882-1210 with seeded random weights instead of files ---- */

@@ -4,11 +4,11 @@
     python tests/golden/make_greedy_fixture.py llama30b_u8 [seed]
 
 Each fixture holds the model shape, the seeds, the 512 prompt token ids, the 128 greedy tokens the
-oracle produces (matmul flavour 2: the 512-token prompt goes through the tensor-core-like flavour,
-every one-token step through the summation order of the HIP decode kernels, so that a decode step
-can be held to the GPU bit for bit; temperature 0.8 as main.cpp:58), and for every
-step the two largest fp16 logits with their token ids and the two largest probabilities, so that
-a mismatch in a GPU run can be attributed to a near-tie.  Only the oracle runs here; nothing from the reference is
+oracle produces (matmul flavour 2: every sum in the order of the HIP kernels -- the matrix cores'
+steps of eight products and the dispatcher's cut of K for the prompt, the lane and wavefront order
+of the decode kernels, v_dot2_f32_f16 for uint8 weights -- so that the whole run can be held to the
+GPU bit for bit; temperature 0.8 as main.cpp:58), and for every step the two largest fp16 logits
+with their token ids and the two largest probabilities.  Only the oracle runs here; nothing from the reference is
 imported or executed.
 """
 import json

@@ -51,6 +51,8 @@ def lib():
         L.orc_dot2_f32_f16.restype = None
         L.orc_attention_decode_kernel_order.argtypes = [vp, vp, vp, vp, i, i, i]
         L.orc_attention_decode_kernel_order.restype = None
+        L.orc_attention_prefill_kernel_order.argtypes = [vp, vp, vp, vp, i, i, i, i, i]
+        L.orc_attention_prefill_kernel_order.restype = None
         L.orc_softmax_logits_kernel_order.argtypes = [vp, vp, i, f]
         L.orc_softmax_logits_kernel_order.restype = None
         L.orc_embed.argtypes = [vp, vp, i, i, vp]
@@ -237,6 +239,17 @@ def exp_f32(x):
     x = np.ascontiguousarray(x, dtype=np.float32)
     out = np.empty_like(x)
     lib().orc_exp_f32(_p(out), _p(x), x.size)
+    return out
+
+
+def attention_prefill_kernel_order(q, k, v, n_heads, start_pos=0):
+    """n_new > 1 rows of q against T = start_pos + n_new cached rows, sums in the order of the HIP kernel"""
+    q, k, v = _f16(q), _f16(k), _f16(v)
+    n_new, dim = q.shape
+    T = k.shape[0]
+    assert T == start_pos + n_new
+    out = np.empty((n_new, dim), dtype=np.float16)
+    lib().orc_attention_prefill_kernel_order(_p(out), _p(q), _p(k), _p(v), n_new, T, start_pos, dim, n_heads)
     return out
 
 

@@ -499,12 +499,15 @@ def test_attention(gpu, n, T):
     assert G.ulp_mismatch(got, ref) < 0.05  # fp32 summation order only
     if start == 0:
         assert G.ulp_mismatch(got[0], v[0]) == 0.0  # causal row 0 sees only itself
-    if n == 1:  # one new token: the oracle restates the kernels' own summation order, every bit
+    # the oracle restates the kernels' own sums (for several rows: the matrix cores' steps), every bit
+    if n == 1:
         assert G.ulp_mismatch(got, O.attention_decode_kernel_order(q, k, v, heads)) == 0.0
+    else:
+        assert G.ulp_mismatch(got, O.attention_prefill_kernel_order(q, k, v, heads, start)) == 0.0
     G.release()
 
 
-@pytest.mark.parametrize("n,T", [(512, 512), (1, 577), (1, 2048), (64, 1024)])
+@pytest.mark.parametrize("n,T", [(512, 512), (1, 577), (1, 2048), (64, 1024), (512, 2048), (33, 1100)])
 def test_attention_llama7b_heads(gpu, n, T):
     """32 heads at dim 4096, the shapes of the benchmark configurations."""
     G = gpu
@@ -522,6 +525,8 @@ def test_attention_llama7b_heads(gpu, n, T):
     assert G.ulp_mismatch(got, ref) < 0.05
     if n == 1:
         assert G.ulp_mismatch(got, O.attention_decode_kernel_order(q, k, v, heads)) == 0.0
+    else:
+        assert G.ulp_mismatch(got, O.attention_prefill_kernel_order(q, k, v, heads, start)) == 0.0
     G.release()
 
 

@@ -93,6 +93,11 @@ def test_matmul_row_independence():
 
 # ------------------------------------------------------------------ flavour 2 (one row in the order of the HIP GEMV kernels)
 def fused_sum_numpy(a, b, c, step):
+    with np.errstate(all="ignore"):
+        return _fused_sum_numpy(a, b, c, step)
+
+
+def _fused_sum_numpy(a, b, c, step):
     """What gfx950 does with fp16 products and an fp32 accumulator (v_dot2_f32_f16: step = 2 = K; the
     matrix cores: steps of 8 over ascending k), restated on its own in float64 from the measured
     samples under tests/golden/.  a, b of shape (n, K) hold halves, c fp32 values.  A half is
@@ -108,7 +113,7 @@ def fused_sum_numpy(a, b, c, step):
             e = np.maximum(e, floor)
         return np.where(v == 0, -10000, e)
 
-    for k0 in range(0, a.shape[1], step):
+    for k0 in range(0, a.shape[1], step):  # (steps without a non-zero product compute with 2^-10024 = 0 and are discarded)
         p = a[:, k0:k0 + step] * b[:, k0:k0 + step]
         e = np.where(p == 0, -10000, expo(a[:, k0:k0 + step], -14) + expo(b[:, k0:k0 + step], -14)).max(1)
         q = np.ldexp(1.0, e - 24)
@@ -370,6 +375,80 @@ def test_attention_decode_kernel_order(T):
         assert np.max(np.abs(got[0, sl].astype(np.float64) - o)) <= 4e-3 * max(np.max(np.abs(o)), 0.05)
     if T == 1:
         assert (got.view(np.uint16) == v[:1].view(np.uint16)).all()  # a single row has probability 1
+
+
+def attention_prefill_numpy(q, k, v, n_heads, start):
+    """Independent restatement of attention_prefill_kernel_order with fused_sum_numpy and exp_f32."""
+    n, dim = q.shape
+    T = k.shape[0]
+    BR = 16 if ((n + 31) // 32) * n_heads < 1024 and T <= 1024 else 32
+    out = np.zeros((n, dim), dtype=np.float16)
+    for h in range(n_heads):
+        sl = slice(h * 128, (h + 1) * 128)
+        for r in range(n):
+            last = min(r // BR * BR + BR, n) - 1
+            Tc = (min(T, last + start + 1) + 63) // 64 * 64
+            vis = min(T, r + start + 1)
+            acc = fused_sum_numpy(np.repeat(q[r:r + 1, sl], vis, 0), k[:vis, sl], np.zeros(vis, dtype=np.float32), 8)
+            sc = np.full(Tc, -np.inf, dtype=np.float16)
+            sc[:vis] = (acc / np.sqrt(np.float32(128.0))).astype(np.float16)
+            x = sc.astype(np.float32)
+            m = x.max()
+            e = O.exp_f32(x - m)
+            pair = (e[0::2] + e[1::2]).astype(np.float32)
+            lanes = np.zeros(64, dtype=np.float32)
+            for i in range(Tc // 2):  # lane i % 64 adds its pairs in ascending order
+                lanes[i % 64] = np.float32(lanes[i % 64] + pair[i])
+            step = 1
+            while step < 64:
+                lanes[::2 * step] = (lanes[::2 * step] + lanes[step::2 * step]).astype(np.float32)
+                step *= 2
+            p = (e / lanes[0]).astype(np.float32).astype(np.float16)
+            vv = np.zeros((Tc, 128), dtype=np.float16)
+            vv[:T] = v[:Tc, sl][:T]
+            o = fused_sum_numpy(np.repeat(p[None, :], 128, 0), np.ascontiguousarray(vv.T), np.zeros(128, dtype=np.float32), 8)
+            out[r, sl] = o.astype(np.float16)
+    return out
+
+
+@pytest.mark.parametrize("n,T", [(5, 5), (3, 130), (40, 70), (17, 17)])
+def test_attention_prefill_kernel_order(n, T):
+    n_heads, dim = 2, 256
+    start = T - n
+    q = f16(RNG.normal(0, 1, (n, dim)))
+    k = f16(RNG.normal(0, 1, (T, dim)))
+    v = f16(RNG.normal(0, 1, (T, dim)))
+    got = O.attention_prefill_kernel_order(q, k, v, n_heads, start)
+    assert (got.view(np.uint16) == attention_prefill_numpy(q, k, v, n_heads, start).view(np.uint16)).all()
+    ref = O.attention(q, k, v, n_heads, start)
+    assert np.max(np.abs(got.astype(np.float64) - ref.astype(np.float64))) <= 2.0 ** -8 * np.max(np.abs(ref.astype(np.float64)))
+    if start == 0:
+        assert (got[0].view(np.uint16) == v[0].view(np.uint16)).all()  # causal row 0 sees only itself
+
+
+def test_context_flavour_2_is_its_operators():
+    """A flavour-2 context is the kernel-order operators chained: a prompt's hidden state equals what
+    the exported pieces give on one layer (so the tests of the pieces carry over to the model)."""
+    cfg = dict(dim=256, multiple_of=128, n_heads=2, n_layers=1, n_vocab=320)
+    om = O.Model(**cfg, seed=2, weight_std=0.05)
+    oc = O.Context(om, context_len=16, temperature=0.8, flavour=2)
+    toks = np.array([3, 100, 7, 250, 9], dtype=np.int16)
+    _, hid, _, _ = oc.next_token(toks, want=True)
+    ffn = om.ffn
+    w = {kind: om.tensor(16 + kind, *((ffn, 256) if kind in (4, 6) else ((256, ffn) if kind == 5 else (256, 256))))[0]
+         for kind in range(7)}
+    x = om.tensor(1, 320, 256)[0][toks]
+    an = fn = np.ones(256, dtype=np.float16)  # synthetic models keep their norm weights at one
+    nx = O.rms_norm(x, an, 1e-6)
+    xq = O.rotary(O.matmul_nt_kernel_order(nx, w[0], n_mats=3), 2)
+    xk = O.rotary(O.matmul_nt_kernel_order(nx, w[1], n_mats=3), 2)
+    xv = O.matmul_nt_kernel_order(nx, w[2], n_mats=3)
+    att = O.attention_prefill_kernel_order(xq, xk, xv, 2, 0)
+    x = O.matmul_nt_kernel_order(att, w[3], beta=1.0, out=x)
+    nx = O.rms_norm(x, fn, 1e-6)
+    up = O.silu_mul(O.matmul_nt_kernel_order(nx, w[4], n_mats=2), O.matmul_nt_kernel_order(nx, w[6], n_mats=2))
+    x = O.matmul_nt_kernel_order(up, w[5], beta=1.0, out=x)
+    assert (x.view(np.uint16) == hid.view(np.uint16)).all()
 
 
 def test_softmax_logits_kernel_order():

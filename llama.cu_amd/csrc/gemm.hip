@@ -20,6 +20,7 @@
 // Both: the K loop carries no vector address arithmetic and no predication; the block index ->
 // tile mapping keeps the tiles that share a slice of W on one XCD (one L2); rows >= M and columns
 // >= N are masked instead of the reference's zeroed "gutter" rows (llama_cu.h:236-242).
+#include <algorithm>
 #include <type_traits>
 
 #include "common.hpp"
@@ -819,25 +820,58 @@ struct partial_sums_t {
   int splits;
 };
 
+// BM x BN tiles of WM x WN wavefronts, the K stages of every tile dealt to `splits` workgroups
+// (gemm_dl_kernel<.., SPLIT = true>), fp32 partial sums in the stream's workspace, then
+// splitk_reduce_kernel -- or the caller's own kernel when `leave` is given.
+template <int BM, int BN, int WM, int WN, bool U8>
+int launch_split(operands_t op, const half_t* A, int M, int K, int N, int block, float beta, hipStream_t st, int splits,
+                 float* part, partial_sums_t* leave = nullptr) {
+  constexpr int KS = 1, NS = 3;
+  constexpr int ROWB = BK * KS * 2;
+  constexpr int DCH = U8 ? BN * (BK * KS / 16) / (64 * WM * WN * KS) : 0;
+  constexpr size_t lds = (size_t)NS * BM * ROWB + (size_t)(U8 ? 2 : NS) * BN * ROWB +
+                         (U8 ? (size_t)NS * (BN * BK * KS + 64 * WM * WN * KS * 4 * DCH) : 0);
+  static_assert(lds <= 160 * 1024, "LDS");
+  const int tiles_m = (M + BM - 1) / BM, tiles_n_per = (N + BN - 1) / BN, tiles_n = tiles_n_per * op.n_mats;
+  op.more.tiles_n_per = op.n_mats > 1 ? tiles_n_per : 0;
+  const size_t mn = (size_t)M * N;
+  auto kernel = gemm_dl_kernel<BM, BN, WM, WN, KS, NS, U8, true>;
+  if constexpr (lds > 64 * 1024) {
+    static bool raised[16] = {};  // per device, once
+    int dev = 0;
+    LCU_HIP(hipGetDevice(&dev));
+    if (!raised[dev & 15]) {
+      LCU_HIP(hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+      raised[dev & 15] = true;
+    }
+  }
+  kernel<<<tiles_m * tiles_n * splits, 64 * WM * WN * KS, lds, st>>>(op.out, A, op.W, op.S, M, K, N, block, beta, tiles_m,
+                                                                     tiles_n, part, splits, op.more);
+  LCU_LAUNCH_CHECK();
+  if (leave) {  // the caller's own kernel adds the partial sums up (fused with what follows the product)
+    leave->part = part;
+    leave->splits = splits;
+  } else {
+    splitk_reduce_kernel<<<dim3((unsigned)((mn + 1023) / 1024), op.n_mats), 256, 0, st>>>(
+        op.out, op.more.out[0], op.more.out[1], part, mn, splits, beta);
+    LCU_LAUNCH_CHECK();
+  }
+  return LCU_OK;
+}
+
 template <int BM, bool U8>
 int launch_skinny(operands_t op, const half_t* A, int M, int K, int N, int block, float beta, hipStream_t st,
                   bool* done, partial_sums_t* leave = nullptr) {
   // a ring of six stages and 128-wide stages with eight wavefronts measured no faster
-  constexpr int BN = 128, WM = 1, WN = 4, KS = 1, NS = 3;
-  constexpr int ROWB = BK * KS * 2;
-  constexpr int DCH = U8 ? BN * (BK * KS / 16) / (256 * KS) : 0;
-  constexpr size_t lds = (size_t)NS * BM * ROWB + (size_t)(U8 ? 2 : NS) * BN * ROWB +
-                         (U8 ? (size_t)NS * (BN * BK * KS + 256 * KS * 4 * DCH) : 0);
-  static_assert(lds <= 160 * 1024, "LDS");
+  constexpr int BN = 128;
   *done = false;
   device_state* ds = current_device_state();
   const workspace_t ws = workspace_for(st);
   if (ds == nullptr || ws.ptr == nullptr) {
     return LCU_OK;
   }
-  const int tiles_m = (M + BM - 1) / BM, tiles_n_per = (N + BN - 1) / BN, tiles_n = tiles_n_per * op.n_mats;
-  op.more.tiles_n_per = op.n_mats > 1 ? tiles_n_per : 0;
-  const int nt_all = K / (BK * KS);
+  const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN * op.n_mats;
+  const int nt_all = K / BK;
   // one workgroup per compute unit and at least four stages each: more, shorter splits only add
   // partial sums (512 workgroups: 16 against 13 us at N = K = 4096)
   int splits = (ds->compute_units + tiles_m * tiles_n - 1) / (tiles_m * tiles_n);
@@ -850,30 +884,26 @@ int launch_skinny(operands_t op, const half_t* A, int M, int K, int N, int block
       (long)tiles_m * tiles_n * splits < ds->compute_units / 2) {
     return LCU_OK;
   }
-  auto kernel = gemm_dl_kernel<BM, BN, WM, WN, KS, NS, U8, true>;
-  if constexpr (lds > 64 * 1024) {
-    static bool raised[16] = {};  // per device, once
-    int dev = 0;
-    LCU_HIP(hipGetDevice(&dev));
-    if (!raised[dev & 15]) {
-      LCU_HIP(hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-      raised[dev & 15] = true;
-    }
+  const int rc = launch_split<BM, BN, 1, 4, U8>(op, A, M, K, N, block, beta, st, splits, (float*)ws.ptr, leave);
+  *done = rc == LCU_OK;
+  return rc;
+}
+
+// Many rows, few 256x128 tiles and a long K (W2 at 512 rows: 64 tiles, K = 11008): with one tile per
+// workgroup most compute units idle, with smaller tiles every workgroup reads more operand bytes per
+// multiply-add than its load path delivers.  So the large tiles stay and the K stages of each are
+// dealt to cus / tiles workgroups, partial sums through the workspace -- when that leaves at least
+// 40 stages per workgroup: the partial sums cost a second launch and M * N * 4 bytes per split each
+// way (K = 11008, N = 4096: 73 -> 59 us with four splits; K = 4096, N = 4096: 25 -> 36 us with two).
+// Returns the number of splits, 0 when the shape does not suit it.
+inline int large_tile_splits(int M, int K, int N, int n_mats, long cus, size_t workspace_bytes) {
+  const long tiles256 = (long)((M + 255) / 256) * ((N + 127) / 128) * n_mats;
+  long splits = std::min<long>(cus / tiles256, 8);
+  splits = std::min<long>(splits, K / BK / 40);
+  if (M <= 64 || splits < 2 || (size_t)splits * M * N * n_mats * sizeof(float) > workspace_bytes) {
+    return 0;
   }
-  float* part = (float*)ws.ptr;
-  kernel<<<tiles_m * tiles_n * splits, 256 * KS, lds, st>>>(op.out, A, op.W, op.S, M, K, N, block, beta, tiles_m, tiles_n,
-                                                            part, splits, op.more);
-  LCU_LAUNCH_CHECK();
-  if (leave) {  // the caller's own kernel adds the partial sums up (fused with what follows the product)
-    leave->part = part;
-    leave->splits = splits;
-  } else {
-    splitk_reduce_kernel<<<dim3((unsigned)((mn + 1023) / 1024), op.n_mats), 256, 0, st>>>(
-        op.out, op.more.out[0], op.more.out[1], part, mn, splits, beta);
-    LCU_LAUNCH_CHECK();
-  }
-  *done = true;
-  return LCU_OK;
+  return (int)splits;
 }
 
 // The direct-to-LDS kernels fetch a thread's fp16 scale as the aligned 4-byte word that holds it:
@@ -1142,6 +1172,16 @@ int dispatch_gemm(operands_t op, const half_t* A, int M, int K, int N, int block
   if (whole_stages) {  // whole stages: the direct-to-LDS kernels
     const long tiles256 = (long)((M + 255) / 256) * ((N + 127) / 128) * nm;
     if (tiles256 >= 160) return launch_dl<256, 128, 4, 2, 1, 3, U8>(op, A, M, K, N, block, beta, st);
+    {
+      device_state* ds = current_device_state();
+      const workspace_t ws = workspace_for(st);
+      if (ds != nullptr && ws.ptr != nullptr) {
+        const int splits = large_tile_splits(M, K, N, op.n_mats, ds->compute_units > 0 ? ds->compute_units : 256, ws.bytes);
+        if (splits > 0) {
+          return launch_split<256, 128, 4, 2, U8>(op, A, M, K, N, block, beta, st, splits, (float*)ws.ptr);
+        }
+      }
+    }
     if constexpr (!U8) {  // uint8 needs a code ring and two W tiles besides: too much LDS for two workgroups
       if (tiles128 >= 256) return launch_dl<128, 128, 2, 2, 1, 2, false>(op, A, M, K, N, block, beta, st);
     }

@@ -432,8 +432,9 @@ inline __m256d mfma_step8(__m256d c, const __m256d* a, const __m256d* sa, const 
 // how K is cut into chains:
 //   * ks == 2 (two groups of wavefronts share a 128-wide K stage): chain 0 takes k with
 //     (k / 64) % 2 == 0, chain 1 the others; the result is chain 0 + chain 1;
-//   * splits > 1 (2..64 rows: K stages of 64 dealt to `splits` workgroups, split s taking stages
-//     [s * n / splits, (s + 1) * n / splits) of n = K / 64): the chains are added in split order.
+//   * splits > 1 (2..64 rows, or few large tiles with a long K: K stages of 64 dealt to `splits`
+//     workgroups, split s taking stages [s * n / splits, (s + 1) * n / splits) of n = K / 64): the
+//     chains are added in split order.
 // plan_gemm restates the dispatcher's choice (dispatch_gemm / launch_skinny) for a device with 256
 // compute units and the 32 MiB workspace of a stream; n_mats is the number of weight matrices of one
 // shape multiplied in one launch (Wq, Wk, Wv: 3; W1, W3: 2).
@@ -472,6 +473,13 @@ gemm_plan plan_gemm(int M, int K, int N, bool u8, int block, int n_mats) {
   if (whole) {
     const long tiles256 = ceil_div(M, 256) * ceil_div(N, 128) * nm;
     if (tiles256 >= 160) return {1, 1};
+    {  // few large tiles and a long K: the K stages of each tile dealt to several workgroups (large_tile_splits)
+      long splits = std::min(cus / tiles256, 8L);
+      splits = std::min(splits, (long)(K / 64 / 40));
+      if (M > 64 && splits >= 2 && (size_t)splits * M * N * nm * sizeof(float) <= workspace) {
+        return {1, (int)splits};
+      }
+    }
     if (!u8 && tiles128 >= 256) return {1, 1};
     if (tiles128 < 256) {
       if (tiles128 >= 160) return {1, 1};

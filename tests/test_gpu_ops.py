@@ -215,7 +215,7 @@ def test_gemm_exact_cases(gpu):
 @pytest.mark.parametrize("M,K,N", [(512, 4096, 4096), (512, 4096, 11008), (512, 11008, 4096), (16, 256, 128),
                                    (130, 384, 70), (512, 256, 5120), (512, 384, 4160), (1024, 256, 4096),
                                    (500, 128, 5100), (40, 384, 300), (4096, 128, 4096), (512, 256, 17920),
-                                   (5, 4096, 4096), (17, 1024, 5000), (32, 11008, 4096), (64, 1024, 4100)])
+                                   (5, 4096, 4096), (17, 1024, 5000), (32, 11008, 4096), (64, 1024, 4100), (512, 17920, 6656)])
 def test_gemm_u8(gpu, M, K, N):
     G = gpu
     x = normal((M, K), 0, 400, 1.0)

@@ -240,7 +240,8 @@ def test_mfma_closed_forms():
                                         ((512, 4096, 4096, False, 3), (1, 1)), ((512, 4096, 11008, False, 2), (1, 1)),
                                         ((32, 11008, 4096, True, 1), (1, 8)), ((2, 4096, 4096, False, 1), (1, 8)),
                                         ((8, 4096, 4096, False, 3), (1, 3)), ((130, 200, 70, False, 1), (2, 1)),
-                                        ((512, 6656, 6656, True, 3), (1, 1)), ((64, 4096, 11008, False, 1), (1, 3))])
+                                        ((512, 6656, 6656, True, 3), (1, 1)), ((64, 4096, 11008, False, 1), (1, 3)),
+                                        ((512, 11008, 4096, False, 1), (1, 4)), ((512, 17920, 6656, True, 1), (1, 2))])
 def test_gemm_plan(shape, plan):
     M, K, N, u8, n_mats = shape
     assert O.gemm_plan(M, K, N, u8, 128, n_mats) == plan

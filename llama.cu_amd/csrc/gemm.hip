@@ -13,8 +13,9 @@
 //     of 256x128, 128x128 or 128x64 with 4 or 8 wavefronts (a second group of four may take the
 //     other half of a 128-wide K stage), chosen by how many tiles the product has; uint8 weights
 //     add a ring of codes and of scales and are turned into fp16 -- exactly fp16((q - 127.5) *
-//     scale), llama_cu.cu:287-289 -- once per block tile; with 2..64 rows the K range is split over
-//     workgroups and a second launch adds the fp32 partial sums (launch_skinny)
+//     scale), llama_cu.cu:287-289 -- once per block tile; with 2..64 rows, and with few large tiles
+//     and a long K, the K range is split over workgroups and a second launch adds the fp32 partial
+//     sums in split order (launch_skinny, large_tile_splits)
 //   gemm_kernel (ragged K): global -> registers -> padded LDS with two LDS buffers and two
 //     register stages, uint8 weights dequantised between the load and the LDS store
 // Both: the K loop carries no vector address arithmetic and no predication; the block index ->
@@ -810,10 +811,6 @@ int launch_dl(operands_t op, const half_t* A, int M, int K, int N, int block, fl
   return LCU_OK;
 }
 
-// Few rows (2 .. 64: short prompts, where the reference takes its 16-row tile, llama_cu.cu:1481-1484):
-// BM x 128 tiles with four wavefronts, the K stages split over enough workgroups to give every
-// compute unit one, fp32 partial sums in the per-device workspace, then splitk_reduce_kernel.
-// Returns LCU_OK with *done = false when the shape does not suit it.
 // where a split-K launch left its partial sums: part[matrix][split][M][N] fp32
 struct partial_sums_t {
   const float* part;
@@ -859,6 +856,9 @@ int launch_split(operands_t op, const half_t* A, int M, int K, int N, int block,
   return LCU_OK;
 }
 
+// Few rows (2 .. 64: short prompts, where the reference takes its 16-row tile, llama_cu.cu:1481-1484):
+// BM x 128 tiles with four wavefronts, the K stages split over enough workgroups to give every
+// compute unit one.  Returns LCU_OK with *done = false when the shape does not suit it.
 template <int BM, bool U8>
 int launch_skinny(operands_t op, const half_t* A, int M, int K, int N, int block, float beta, hipStream_t st,
                   bool* done, partial_sums_t* leave = nullptr) {

@@ -222,6 +222,101 @@ def test_batched_decode_vs_oracle(gpu, q_type):
     gm.close()
 
 
+class BatchOracle:
+    """One step of several sequences at once, built from the oracle's kernel-order operators the way
+    host/batch.cpp chains the fused device kernels: the rows of all sequences go through every matrix
+    product together (what cuts K there depends on the number of rows and of matrices per launch),
+    everything else is per sequence.  Prompts go through the sequence's own flavour-2 context, whose
+    cache this class reads and extends."""
+
+    def __init__(self, om, cfg, context_len, temperature):
+        self.om, self.cfg, self.T, self.temp = om, cfg, context_len, temperature
+        self.u8 = cfg.get("q_type", 0) == 1
+        dim, ffn, vocab = cfg["dim"], om.ffn, cfg["n_vocab"]
+        shapes = {0: (dim, dim), 1: (dim, dim), 2: (dim, dim), 3: (dim, dim), 4: (ffn, dim), 5: (dim, ffn), 6: (ffn, dim)}
+        self.w = [[om.tensor(16 + 16 * l + k, *shapes[k]) for k in range(7)] for l in range(cfg["n_layers"])]
+        self.emb = om.tensor(1, vocab, dim)
+        self.out = om.tensor(2, vocab, dim)
+        self.ones = np.ones(dim, dtype=np.float16)  # synthetic models keep their norm weights at one
+        self.k, self.v, self.pos = {}, {}, {}
+
+    def mm(self, x, w, n_mats=1, beta=0.0, out=None):
+        if self.u8:
+            return O.matmul_nt_kernel_order(x, codes=w[0], scales=w[1], block=128, beta=beta, out=out, n_mats=n_mats)
+        return O.matmul_nt_kernel_order(x, w[0], beta=beta, out=out, n_mats=n_mats)
+
+    def adopt(self, b, oc, n_tokens):
+        """take over sequence b from a context that has seen n_tokens"""
+        L, dim = self.cfg["n_layers"], self.cfg["dim"]
+        self.k[b] = np.zeros((L, self.T, dim), dtype=np.float16)
+        self.v[b] = np.zeros((L, self.T, dim), dtype=np.float16)
+        for l in range(L):
+            kk, vv = oc.kv(l, n_tokens)
+            self.k[b][l, :n_tokens], self.v[b][l, :n_tokens] = kk, vv
+        self.pos[b] = n_tokens
+
+    def step(self, seqs, tokens):
+        cfg, H = self.cfg, self.cfg["n_heads"]
+        ids = np.array(tokens, dtype=np.int16)
+        x = O.embed_u8(ids, self.emb[0], self.emb[1], 128) if self.u8 else O.embed(ids, self.emb[0])
+        for l in range(cfg["n_layers"]):
+            w = self.w[l]
+            nx = O.rms_norm(x, self.ones, 1e-6)
+            q, k, v = (self.mm(nx, w[i], n_mats=3) for i in range(3))
+            att = np.empty_like(x)
+            for r, b in enumerate(seqs):
+                t = self.pos[b]
+                qr = O.rotary(q[r:r + 1], H, t)
+                self.k[b][l, t] = O.rotary(k[r:r + 1], H, t)[0]
+                self.v[b][l, t] = v[r]
+                att[r] = O.attention_decode_kernel_order(qr, self.k[b][l, :t + 1], self.v[b][l, :t + 1], H)[0]
+            x = self.mm(att, w[3], beta=1.0, out=x)
+            nx = O.rms_norm(x, self.ones, 1e-6)
+            up = O.silu_mul(self.mm(nx, w[4], n_mats=2), self.mm(nx, w[6], n_mats=2))
+            x = self.mm(up, w[5], beta=1.0, out=x)
+        logits = self.mm(O.rms_norm(x, self.ones, 1e-6), self.out)
+        probs = np.stack([O.softmax_logits_kernel_order(logits[r], self.temp) for r in range(len(seqs))])
+        for b in seqs:
+            self.pos[b] += 1
+        return logits, probs, [O.argmax_first(p) for p in probs]
+
+
+@pytest.mark.parametrize("cfg,lens", [(dict(dim=512, multiple_of=128, n_heads=4, n_layers=3, n_vocab=2048), (19, 3, 40)),
+                                       (dict(dim=512, multiple_of=128, n_heads=4, n_layers=3, n_vocab=2048, q_type=1,
+                                             qblock=128), (5, 33, 2, 70, 1)),
+                                       (dict(dim=4096, multiple_of=256, n_heads=32, n_layers=2, n_vocab=32000),
+                                        (9, 64, 3, 17, 30, 5, 12, 40))])
+def test_batched_decode_bit_exact_against_kernel_order_oracle(gpu, cfg, lens):
+    """llama_batch_context against the kernel-order oracle, every bit: the sequences' prompts, then
+    steps of all sequences together (eager, captured, replayed), logits, probabilities and tokens."""
+    G = gpu
+    std = 0.05 if cfg["dim"] == 512 else 0.02
+    om = O.Model(**cfg, seed=21, weight_std=std)
+    gm = G.P.Model(**cfg, seed=21, weight_std=std)
+    rng = np.random.default_rng(3)
+    B, ctx = len(lens), 96
+    bo = BatchOracle(om, cfg, ctx, 0.8)
+    bc = G.P.BatchContext(gm, B, context_len=ctx, temperature=0.8)
+    last = []
+    for b, n in enumerate(lens):
+        pr = rng.integers(0, cfg["n_vocab"], n).astype(np.int16)
+        oc = O.Context(om, context_len=ctx, temperature=0.8, flavour=2)
+        otok = oc.next_token(pr)
+        assert bc.next_token(b, pr) == otok, b
+        bo.adopt(b, oc, n)
+        oc.close()
+        last.append(otok)
+    for k in range(5):
+        logits, probs, toks = bo.step(list(range(B)), last)
+        got = bc.next_tokens(last)
+        assert G.ulp_mismatch(bc.logits(), logits) == 0.0, k
+        assert G.ulp_mismatch(bc.probs(), probs) == 0.0, k
+        assert list(got) == toks, k
+        last = toks
+    bc.close()
+    gm.close()
+
+
 def test_batched_decode_with_a_long_and_a_short_sequence(gpu):
     """One sequence beyond 1024 cached rows (where a single context switches its attention form and the batch
     raises its bound), one at the start: both follow their own single-sequence contexts."""

@@ -282,6 +282,46 @@ def test_gemm_multi_matches_separate_calls(gpu, M, K, N, count):
     G.release()
 
 
+def test_gemm_dispatch_sweep_bit_exact(gpu):
+    """Seventy seeded shapes across the dispatcher's branches (few and many rows, K in whole stages or
+    ragged, tile counts on both sides of every threshold, one to three matrices per launch, fp16 and
+    uint8): the oracle's restatement of the cut of K must give the device's bits on all of them."""
+    G = gpu
+    L = G.L()
+    VP = G.B.vp
+    rng = np.random.default_rng(77)
+    plans = set()
+    for case in range(70):
+        M = int(rng.choice([2, 7, 32, 33, 64, 65, 100, 256, 300, 512, 700, 1100]))
+        K = int(rng.choice([64, 128, 136, 256, 384, 640, 1024, 2560, 5120]))
+        N = int(rng.choice([24, 128, 1000, 2048, 4096, 5120, 8200, 11008, 17920]))
+        nm = int(rng.choice([1, 1, 2, 3]))
+        u8 = bool(rng.integers(0, 2)) and K % 128 == 0
+        if M * K * N * nm > 2.5e10:
+            K = 128
+        x = normal((M, K), 5, 3 * case, 1.0)
+        ws = [normal((N, K), 5, 3 * case + 1 + g, 0.02) for g in range(nm)]
+        xd = G.dev_keep(x)
+        outs = [G.empty((M, N)) for _ in range(nm)]
+        out_arr = (VP * nm)(*[o.ptr for o in outs])
+        if u8:
+            q = [O.quantize_absmax_u8(w, 128) for w in ws]
+            cd, sd = [G.dev_keep(c) for c, _ in q], [G.dev_keep(sc) for _, sc in q]
+            G.B.check(L.lcu_gemm_f16u8_nt_multi(out_arr, xd.ptr, (VP * nm)(*[c.ptr for c in cd]), (VP * nm)(*[sc.ptr for sc in sd]),
+                                                nm, M, K, N, 128, 0.0, None))
+            want = [O.matmul_nt_kernel_order(x, codes=c, scales=sc, block=128, n_mats=nm) for c, sc in q]
+        else:
+            wd = [G.dev_keep(w) for w in ws]
+            G.B.check(L.lcu_gemm_f16_nt_multi(out_arr, xd.ptr, (VP * nm)(*[w.ptr for w in wd]), nm, M, K, N, 0.0, None))
+            want = [O.matmul_nt_kernel_order(x, w, n_mats=nm) for w in ws]
+        plan = O.gemm_plan(M, K, N, u8, 128, nm)
+        plans.add(plan)
+        for g in range(nm):
+            assert G.ulp_mismatch(G.host(outs[g], (M, N)), want[g]) == 0.0, (case, M, K, N, nm, u8, plan, g)
+        G.release()
+    assert len(plans) >= 6, plans  # single chains, two groups per stage, several depths of split
+
+
 def test_streams_own_their_workspace(gpu):
     """Split-K products (2..64 rows) keep fp32 partial sums in scratch memory.  Every stream made by
     lcu_stream_create has a workspace of its own, so two host threads driving two streams at once

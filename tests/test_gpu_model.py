@@ -398,6 +398,14 @@ def test_prompt_longer_than_the_multi_row_attention_reaches(gpu):
     ok, ov = oc.kv(0, 2150)
     gk, gv = gc.kv(0, 2150)
     assert G.max_abs_rel(gk, ok) <= TOL and G.max_abs_rel(gv, ov) <= TOL
+    # the kernel-order oracle fed the same pieces (2048 rows, then one token at a time): every bit
+    ko = O.Context(om, context_len=2200, temperature=0.8, flavour=2)
+    ko.next_token(toks[:2048])
+    for t in toks[2048:2150]:
+        ktok, _, klogits, _ = ko.next_token(np.array([t], dtype=np.int16), want=True)
+    assert G.ulp_mismatch(gc.logits(), klogits) == 0.0 and gtok == ktok
+    kk, kv = ko.kv(0, 2150)
+    assert G.ulp_mismatch(gk, kk) == 0.0 and G.ulp_mismatch(gv, kv) == 0.0
     gc.close()
     gm.close()
 

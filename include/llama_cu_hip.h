@@ -59,6 +59,8 @@ int lcu_d2h(void* dst_host, const void* src_dev, size_t bytes, void* stream);   
 int lcu_d2d(void* dst_dev, const void* src_dev, size_t bytes, void* stream);
 int lcu_stream_create(void** out_stream);
 int lcu_stream_destroy(void* stream);
+/* bounded in-launch waits that ran out on this stream's workspace so far (0 in any healthy run) */
+int lcu_sync_timeouts(void* stream, unsigned* out_count);
 int lcu_sync(void* stream);                                                     /* NULL = whole device */
 /* HIP graph capture of the launches made on `stream` between begin and end; every lcu_* kernel
  * entry point may be captured (none of them records a memset node or allocates).  No counterpart
@@ -159,6 +161,19 @@ int lcu_attention(void* out_dev, const void* q_dev, const void* k_dev, const voi
  * 1024 while the position allows it.  Uses the stream's workspace when max_T > 1024. */
 int lcu_attention_decode(void* out_dev, const void* q_dev, const void* k_dev, const void* v_dev,
                          const void* pos_dev, int max_T, int dim, int n_heads, void* stream);
+
+/* lcu_attention_decode with the work of a head spread over eight workgroups, which hand their scores
+ * to one another inside the launch through the stream's workspace (same bits as
+ * lcu_attention_decode).  Every score travels with the launch's epoch, *seq_dev << 10 | salt: seq_dev is a device
+ * uint32 that the caller changes (counts up) before every run of the call, also before every replay
+ * of a graph that holds it; salt (0..1023) tells the calls of one such run apart (the layer index).
+ * Two consecutive launches on a stream must never have the same epoch.  A hand-over that does not
+ * arrive (it cannot on an otherwise idle device) is given up after a bounded wait and counted:
+ * lcu_sync_timeouts.  No counterpart in the reference (its score tensor goes through memory
+ * between three launches, llama_cu.cu:1161-1171). */
+int lcu_attention_decode_spread(void* out_dev, const void* q_dev, const void* k_dev, const void* v_dev,
+                                const void* pos_dev, const void* seq_dev, int salt, int max_T, int dim, int n_heads,
+                                void* stream);
 
 /* ---- one decode step of several sequences (batching is a TODO of the reference, README.md:34):
  * the GEMMs take the n_seq rows as M; these three handle what differs per sequence.  The caches

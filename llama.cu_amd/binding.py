@@ -72,6 +72,8 @@ SIGNATURES = {
     "lcu_attention": (i32, [vp, vp, vp, vp, i32, i32, i32, i32, i32, vp]),
     "lcu_decode_qkv": (i32, [vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, i32, i32, i32, i32, vp, f32, vp, i32, vp]),
     "lcu_attention_decode": (i32, [vp, vp, vp, vp, vp, i32, i32, i32, vp]),
+    "lcu_attention_decode_spread": (i32, [vp, vp, vp, vp, vp, vp, i32, i32, i32, i32, vp]),
+    "lcu_sync_timeouts": (i32, [vp, vp]),
     "lcu_graph_begin_capture": (i32, [vp]),
     "lcu_graph_end_capture": (i32, [vp, C.POINTER(vp)]),
     "lcu_graph_launch": (i32, [vp, vp]),

@@ -16,6 +16,8 @@
 // v_mfma_f32_16x16x32_f16 into an LDS score strip [rows][T], softmax in LDS, P.V by MFMA with V
 // staged row-major in LDS; the next 64-row chunk of K or V is in flight while the current one is
 // multiplied.
+#include <atomic>
+
 #include "common.hpp"
 
 using namespace lcu;
@@ -266,6 +268,199 @@ __global__ __launch_bounds__(256) void dec_softmax_pv_kernel(half_t* __restrict_
     for (int g = 0; g < 64; ++g) o += gsum[g][tid];
     out[h * HD + slice * PV_COLS + tid] = round_f16(o);  // 529
   }
+}
+
+// ---- decode attention spread over eight workgroups per head, one launch -------------------------
+// A compute unit fetches cold cache rows at about 30 GB/s (its count of outstanding misses, not its
+// 120 GB/s path, is the limit), so one workgroup per head spends 5 of its 9 us waiting for the
+// head's K alone.  Here eight 256-thread workgroups share a head: each takes every eighth block of
+// 16 cached rows for the scores and 16 of the head's 128 columns for the weighted sum.  The
+// softmax needs the whole row of scores, so the workgroups of a head hand theirs to one another
+// inside the launch:
+//   * a score travels as an 8-byte word {fp16 score, epoch of the launch}, written with one
+//     device-scope store (through to memory) and read with device-scope loads, so the hand-over
+//     does not depend on which caches the workgroups share and needs no flag, fence or reset: a
+//     reader asks for the words it needs until every one carries this launch's epoch, a value that
+//     no earlier launch can have left in them (host-drawn epochs have the top bit set and count
+//     up; device epochs are step counter << 10 | salt with the top bit clear);
+//   * the wait is bounded: the eight workgroups of a head have neighbouring indices, all are
+//     resident at once on any idle device (256 threads, 7 KB of LDS), and a wait that runs out
+//     anyway counts itself in the stream's sync area (lcu_sync_timeouts) and goes on;
+//   * workgroup b runs on XCD b % 8 (round-robin dispatch), so b = xcd + 8 * (slice + 8 * i) keeps
+//     a head's workgroups on one XCD, where they share the L2 lines of the head's K and V rows.
+// Every sum is associated as in decode_attention_kernel (16 lanes x 8 elements per score; the
+// reference's 256-thread softmax; row groups g, g + 64, ... then the 64 groups in order), so the
+// bits are the same.  NJ: the row bound is 256 * NJ.
+constexpr int SPREAD = 8;
+constexpr int SPREAD_SPIN_LIMIT = 1 << 16;
+
+// the wait for it is the caller's (s_waitcnt vmcnt(0) after the last of a group)
+__device__ __forceinline__ uint64_t request_u64_device_scope(const uint64_t* p) {
+  uint64_t v;
+  asm volatile("global_load_dwordx2 %0, %1, off sc0 sc1" : "=v"(v) : "v"(p) : "memory");
+  return v;
+}
+
+template <int NJ>
+__global__ __launch_bounds__(256) void decode_attention_spread_kernel(
+    half_t* __restrict__ out, const half_t* __restrict__ q, const half_t* __restrict__ k, const half_t* __restrict__ v,
+    int T_cap, int dim, int n_heads, const int* __restrict__ pos_dev, uint64_t* __restrict__ scores,
+    const uint32_t* __restrict__ seq_dev, uint32_t epoch, uint32_t* __restrict__ timeouts) {
+  __shared__ half_t sc[256 * NJ];  // fp16 probabilities
+  __shared__ float gsum[64][17];
+  __shared__ __attribute__((aligned(16))) float red[8];
+  const int b = blockIdx.x, tid = threadIdx.x;
+  const int slice = (b >> 3) & 7, h = (b & 7) + 8 * (b >> 6);
+  if (h >= n_heads) return;
+  int T = T_cap;
+  if (pos_dev) T = min(max(*pos_dev + 1, 1), T_cap);
+  if (seq_dev) epoch = (epoch | (*seq_dev << 10)) & 0x7fffffffu;
+
+  // ---- scores of rows slice * 16 + grp + 128 f, llama_cu.cu:400-428
+  const int sub = tid & 15, grp = tid >> 4;
+  const half_t* kh = k + h * HD + sub * 8;
+  uint64_t* srow = scores + (size_t)h * T_cap;
+  const float denom = sqrtf((float)HD);
+  half8_t qh;
+  for (int p0 = 0; p0 < T; p0 += 1024) {
+    half8_t kv[8];
+#pragma unroll
+    for (int f = 0; f < 8; ++f) {
+      const int p = p0 + slice * 16 + grp + 128 * f;
+      kv[f] = p < T ? __builtin_nontemporal_load(reinterpret_cast<const half8_t*>(kh + (size_t)p * dim))
+                    : (half8_t)(0.0f);
+    }
+    if (p0 == 0) qh = *reinterpret_cast<const half8_t*>(q + h * HD + sub * 8);
+#pragma unroll
+    for (int f = 0; f < 8; ++f) {
+      const int p = p0 + slice * 16 + grp + 128 * f;
+      float s = 0.0f;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) s = fmaf((float)qh[e], (float)kv[f][e], s);
+      s = row16_sum(s);
+      if (sub == 0 && p < T) {
+        const half_t val = round_f16(s / denom);  // 425
+        const uint64_t word = ((uint64_t)epoch << 32) | __builtin_bit_cast(unsigned short, val);
+        __hip_atomic_store(srow + p, word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+    }
+  }
+  // the first 1024 rows of this workgroup's 16 columns of V: 4 lanes x 8 bytes per row, row group
+  // vg takes rows vg + 64 f; on their way during the hand-over and the softmax
+  const int vsub = tid & 3, vg = tid >> 2;
+  const half_t* vh = v + h * HD + slice * 16 + vsub * 4;
+  half4_t vv[16];
+#pragma unroll
+  for (int f = 0; f < 16; ++f) {
+    const int p = vg + 64 * f;
+    vv[f] = p < T ? *reinterpret_cast<const half4_t*>(vh + (size_t)p * dim) : (half4_t)(0.0f);
+  }
+
+  // ---- hand-over and softmax_rows, llama_cu.cu:433-499: thread t owns elements t, t + 256, ... as
+  // there; every wavefront asks for its elements until all of them are this launch's
+  float x[NJ];
+  {
+    uint64_t raw[NJ];
+    int spins = 0;
+    while (true) {
+#pragma unroll
+      for (int j = 0; j < NJ; ++j) {
+        raw[j] = tid + 256 * j < T ? request_u64_device_scope(srow + tid + 256 * j) : ((uint64_t)epoch << 32) | 0xfc00u;
+      }
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      bool stale = false;
+#pragma unroll
+      for (int j = 0; j < NJ; ++j) {
+        asm volatile("" : "+v"(raw[j]));  // read only after the wait
+        stale |= (uint32_t)(raw[j] >> 32) != epoch;
+      }
+      if (__builtin_amdgcn_ballot_w64(stale) == 0) break;
+      if (++spins > SPREAD_SPIN_LIMIT) {
+        if ((tid & 63) == 0) atomicAdd(timeouts, 1u);
+        break;
+      }
+      __builtin_amdgcn_s_sleep(1);
+    }
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) x[j] = (float)__builtin_bit_cast(half_t, (unsigned short)raw[j]);
+  }
+  float m = x[0];
+#pragma unroll
+  for (int j = 1; j < NJ; ++j) m = fmaxf(m, x[j]);
+  m = block256_max_dpp(m, red);
+  float s = 0.0f;
+#pragma unroll
+  for (int j = 0; j < NJ; ++j) {
+    if (tid + 256 * j < T) {
+      x[j] = exp_ieee(x[j] - m);
+      s += x[j];
+    }
+  }
+  const float total = block256_sum_ref_order_dpp(s, red);
+#pragma unroll
+  for (int j = 0; j < NJ; ++j) {
+    if (tid + 256 * j < T) sc[tid + 256 * j] = round_f16(x[j] / total);  // 497
+  }
+  __syncthreads();
+
+  // ---- matmul_qkv, llama_cu.cu:511-531, for this workgroup's 16 columns
+  float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+  for (int p0 = 0; p0 < T; p0 += 1024) {
+    if (p0 > 0) {
+#pragma unroll
+      for (int f = 0; f < 16; ++f) {
+        const int p = p0 + vg + 64 * f;
+        vv[f] = p < T ? *reinterpret_cast<const half4_t*>(vh + (size_t)p * dim) : (half4_t)(0.0f);
+      }
+    }
+#pragma unroll
+    for (int f = 0; f < 16; ++f) {
+      const int p = p0 + vg + 64 * f;
+      if (p < T) {
+        const float prob = (float)sc[p];
+#pragma unroll
+        for (int c = 0; c < 4; ++c) acc[c] = fmaf(prob, (float)vv[f][c], acc[c]);
+      }
+    }
+  }
+#pragma unroll
+  for (int c = 0; c < 4; ++c) gsum[vg][vsub * 4 + c] = acc[c];
+  __syncthreads();
+  if (tid < 16) {
+    float o = 0.0f;
+#pragma unroll
+    for (int g = 0; g < 64; ++g) o += gsum[g][tid];
+    out[h * HD + slice * 16 + tid] = round_f16(o);  // 529
+  }
+}
+
+// seq_dev == nullptr: the epoch is a number the host draws per launch (never under stream capture:
+// a replay would repeat it); else it comes from *seq_dev, which the caller changes before every
+// run, and `salt`.  The score words live in the exchange area behind the stream's workspace.
+int launch_decode_attention_spread(half_t* out, const half_t* q, const half_t* k, const half_t* v, const int* pos_dev,
+                                   int T_cap, int dim, int n_heads, const workspace_t& ws, const uint32_t* seq_dev,
+                                   uint32_t salt, hipStream_t s) {
+  static std::atomic<uint32_t> host_epoch{1};
+  uint32_t epoch = salt & 1023u;
+  if (seq_dev == nullptr) {
+    epoch = host_epoch.fetch_add(1) | 0x80000000u;
+  }
+  const int grid = (n_heads + 7) / 8 * 8 * SPREAD;
+  uint64_t* scores = reinterpret_cast<uint64_t*>(ws.sync + SYNC_EXCHANGE);
+  static_assert(SYNC_WORDS - SYNC_EXCHANGE >= MAX_HEADS * MAX_T_DECODE * 2, "exchange area");
+  uint32_t* timeouts = ws.sync + SYNC_TIMEOUTS;
+  if (T_cap <= 1024) {
+    decode_attention_spread_kernel<4><<<grid, 256, 0, s>>>(out, q, k, v, T_cap, dim, n_heads, pos_dev, scores, seq_dev,
+                                                            epoch, timeouts);
+  } else if (T_cap <= 2048) {
+    decode_attention_spread_kernel<8><<<grid, 256, 0, s>>>(out, q, k, v, T_cap, dim, n_heads, pos_dev, scores, seq_dev,
+                                                            epoch, timeouts);
+  } else {
+    decode_attention_spread_kernel<16><<<grid, 256, 0, s>>>(out, q, k, v, T_cap, dim, n_heads, pos_dev, scores, seq_dev,
+                                                             epoch, timeouts);
+  }
+  LCU_LAUNCH_CHECK();
+  return LCU_OK;
 }
 
 // scores: n_heads x T_cap halves of scratch (only touched when T_cap > SINGLE_LAUNCH_MAX_T)
@@ -543,6 +738,13 @@ int lcu_attention(void* out_dev, const void* q_dev, const void* k_dev, const voi
     LCU_REQUIRE(T <= MAX_T_DECODE, "lcu_attention: T %d exceeds %d", T, MAX_T_DECODE);
     const workspace_t ws = workspace_for(s);
     LCU_REQUIRE((size_t)n_heads * T * sizeof(half_t) <= ws.bytes, "lcu_attention: workspace too small");
+    hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+    if (s != nullptr) LCU_HIP(hipStreamIsCapturing(s, &capturing));
+    if (capturing == hipStreamCaptureStatusNone && ws.sync != nullptr) {
+      // the epoch of this launch is drawn on the host, so the launch must not be replayed
+      return launch_decode_attention_spread((half_t*)out_dev, (const half_t*)q_dev, (const half_t*)k_dev,
+                                            (const half_t*)v_dev, nullptr, T, dim, n_heads, ws, nullptr, 0, s);
+    }
     return launch_decode_attention((half_t*)out_dev, (const half_t*)q_dev, (const half_t*)k_dev, (const half_t*)v_dev,
                                    nullptr, T, dim, n_heads, (half_t*)ws.ptr, s);
   }
@@ -590,6 +792,25 @@ int lcu_attention_decode(void* out_dev, const void* q_dev, const void* k_dev, co
   LCU_REQUIRE((size_t)n_heads * max_T * sizeof(half_t) <= ws.bytes, "lcu_attention_decode: workspace too small");
   return launch_decode_attention((half_t*)out_dev, (const half_t*)q_dev, (const half_t*)k_dev, (const half_t*)v_dev,
                                  (const int*)pos_dev, max_T, dim, n_heads, (half_t*)ws.ptr, as_stream(stream));
+}
+
+int lcu_attention_decode_spread(void* out_dev, const void* q_dev, const void* k_dev, const void* v_dev,
+                                const void* pos_dev, const void* seq_dev, int salt, int max_T, int dim, int n_heads,
+                                void* stream) {
+  LCU_REQUIRE(out_dev && q_dev && k_dev && v_dev && pos_dev && seq_dev, "lcu_attention_decode_spread: null pointer");
+  LCU_REQUIRE(n_heads > 0 && n_heads <= MAX_HEADS && dim == n_heads * HD,
+              "lcu_attention_decode_spread: dim %d / heads %d unsupported (head_dim must be 128, at most %d heads)", dim,
+              n_heads, MAX_HEADS);
+  LCU_REQUIRE(max_T > 0 && max_T <= MAX_T_DECODE, "lcu_attention_decode_spread: max_T %d outside 1..%d", max_T,
+              MAX_T_DECODE);
+  LCU_REQUIRE(salt >= 0 && salt < 1024, "lcu_attention_decode_spread: salt %d outside 0..1023", salt);
+  const workspace_t ws = workspace_for(as_stream(stream));
+  if (ws.ptr == nullptr || ws.sync == nullptr) {
+    return set_error(LCU_E_NOINIT, "lcu_attention_decode_spread: lcu_init has not run on this device");
+  }
+  return launch_decode_attention_spread((half_t*)out_dev, (const half_t*)q_dev, (const half_t*)k_dev,
+                                        (const half_t*)v_dev, (const int*)pos_dev, max_T, dim, n_heads, ws,
+                                        (const uint32_t*)seq_dev, (uint32_t)salt, as_stream(stream));
 }
 
 int lcu_attention_decode_static(void* out_dev, const void* q_dev, const void* k_dev, const void* v_dev, int T, int dim,

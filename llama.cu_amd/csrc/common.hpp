@@ -45,6 +45,7 @@ struct device_state {
   int compute_units = 0;
   void* workspace = nullptr;  // scratch of the default stream and of streams this library did not create
   size_t workspace_bytes = 0;
+  uint32_t* workspace_sync = nullptr;
 };
 device_state* current_device_state();
 
@@ -56,7 +57,15 @@ device_state* current_device_state();
 struct workspace_t {
   void* ptr = nullptr;
   size_t bytes = 0;
+  // SYNC_WORDS zero-initialised uint32 behind the scratch, never used as scratch: what workgroups
+  // of one launch hand to one another (decode attention spread over several workgroups per head).
+  // Words 0 .. SYNC_TIMEOUTS are counters; from SYNC_EXCHANGE on, 64 heads x 4096 rows of 8-byte
+  // {value, epoch} words, which no other operator may write: a reader trusts a word by its epoch.
+  uint32_t* sync = nullptr;
 };
+constexpr int SYNC_EXCHANGE = 2048;
+constexpr int SYNC_WORDS = SYNC_EXCHANGE + 64 * 4096 * 2;
+constexpr int SYNC_TIMEOUTS = SYNC_EXCHANGE - 1;  // word that counts bounded waits which ran out
 workspace_t workspace_for(hipStream_t stream);
 
 // fp32 -> fp16, round to nearest even, as a separate step.  Written through an opaque register so
@@ -152,6 +161,58 @@ __device__ __forceinline__ float block256_sum_ref_order(float v, float* red) {
     w += __shfl_xor(w, off, WAVE);
   }
   return w;
+}
+
+// The same sum, same association, with the xor steps 8, 4, 2, 1 as data-parallel-primitive moves
+// (xor 4: a shift by four lanes to the left for lanes 0-3 and 8-11 of a row, to the right for the
+// others) and the eight group sums added in registers by every thread: the reference's xor steps
+// 4, 2, 1 over lanes holding r0..r7 leave ((r0 + r4) + (r2 + r6)) + ((r1 + r5) + (r3 + r7)) in lane 0
+// and, additions being commutative, the same bits in the other seven.  One ds_bpermute and one
+// barrier pair instead of eight and two.
+__device__ __forceinline__ float block256_sum_ref_order_dpp(float v, float* red) {
+  v += __shfl_xor(v, 16, WAVE);
+  v += dpp_f32<0x128>(v);  // row_ror:8 = xor 8 inside a row of 16
+  {
+    const int vi = __builtin_bit_cast(int, v);
+    int t = __builtin_amdgcn_update_dpp(0, vi, 0x104, 0xF, 0x5, false);  // row_shl:4 into lanes 0-3, 8-11
+    t = __builtin_amdgcn_update_dpp(t, vi, 0x114, 0xF, 0xA, false);      // row_shr:4 into lanes 4-7, 12-15
+    v += __builtin_bit_cast(float, t);
+  }
+  v += dpp_f32<0x4E>(v);  // quad_perm [2,3,0,1]
+  v += dpp_f32<0xB1>(v);  // quad_perm [1,0,3,2]
+  const int tid = threadIdx.x;
+  __syncthreads();  // protects `red` against a previous use
+  if ((tid & 31) == 0) {
+    red[tid >> 5] = v;
+  }
+  __syncthreads();
+  const float4_t lo = *reinterpret_cast<const float4_t*>(red), hi = *reinterpret_cast<const float4_t*>(red + 4);
+  return ((lo[0] + hi[0]) + (lo[2] + hi[2])) + ((lo[1] + hi[1]) + (lo[3] + hi[3]));
+}
+
+// maximum over a wavefront with data-parallel-primitive moves (the order of a maximum is free)
+__device__ __forceinline__ float wave_max_dpp(float v) {
+  v = fmaxf(v, dpp_f32<0xB1>(v));
+  v = fmaxf(v, dpp_f32<0x4E>(v));
+  v = fmaxf(v, dpp_f32<0x141>(v));
+  v = fmaxf(v, dpp_f32<0x140>(v));
+  const int vi = __builtin_bit_cast(int, v);
+  const float r0 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(vi, 0));
+  const float r1 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(vi, 16));
+  const float r2 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(vi, 32));
+  const float r3 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(vi, 48));
+  return fmaxf(fmaxf(r0, r1), fmaxf(r2, r3));
+}
+__device__ __forceinline__ float block256_max_dpp(float v, float* red) {
+  v = wave_max_dpp(v);
+  const int tid = threadIdx.x;
+  __syncthreads();
+  if ((tid & 63) == 0) {
+    red[tid >> 6] = v;
+  }
+  __syncthreads();
+  const float4_t r = *reinterpret_cast<const float4_t*>(red);
+  return fmaxf(fmaxf(r[0], r[1]), fmaxf(r[2], r[3]));
 }
 
 __device__ __forceinline__ float block256_max(float v, float* red) {

@@ -15,11 +15,34 @@ namespace {
 __global__ __launch_bounds__(256) void rmsnorm_kernel(half_t* out, const half_t* in,
                                                       const half_t* __restrict__ weights, int cols, float eps) {
   extern __shared__ half_t xs[];  // the row, so that it is read from memory once, with 16-byte loads
-  __shared__ float red[8];
+  __shared__ __attribute__((aligned(16))) float red[8];
   const half_t* x = in + (size_t)blockIdx.x * cols;
   half_t* y = out + (size_t)blockIdx.x * cols;
   const bool vec = (cols % 8) == 0;
-  if (vec) {
+  // rows of up to 8192 elements (every model width): up to four pieces per thread, the weights
+  // requested together with the row, so the kernel has one memory round trip before its stores;
+  // longer rows take the general loops below
+  constexpr int P = 4;
+  const bool few = vec && cols <= P * 256 * 8;
+  half8_t wp[P];
+  if (few) {
+    uint4 xp[P];
+#pragma unroll
+    for (int j = 0; j < P; ++j) {
+      const int i = (threadIdx.x + 256 * j) * 8;
+      xp[j] = i < cols ? *reinterpret_cast<const uint4*>(x + i) : make_uint4(0, 0, 0, 0);
+    }
+#pragma unroll
+    for (int j = 0; j < P; ++j) {
+      const int i = (threadIdx.x + 256 * j) * 8;
+      wp[j] = i < cols ? *reinterpret_cast<const half8_t*>(weights + i) : (half8_t)(0.0f);
+    }
+#pragma unroll
+    for (int j = 0; j < P; ++j) {
+      const int i = (threadIdx.x + 256 * j) * 8;
+      if (i < cols) *reinterpret_cast<uint4*>(xs + i) = xp[j];
+    }
+  } else if (vec) {
     for (int i = threadIdx.x * 8; i < cols; i += 256 * 8) {
       *reinterpret_cast<uint4*>(xs + i) = *reinterpret_cast<const uint4*>(x + i);
     }
@@ -28,13 +51,37 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(half_t* out, const half_t*
   }
   __syncthreads();
   float s = 0.0f;
-  for (int i = threadIdx.x; i < cols; i += 256) {
+  // eight LDS reads in flight at a time; the additions stay in ascending order
+  int i = threadIdx.x;
+  for (; i + 7 * 256 < cols; i += 8 * 256) {
+    float v[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) v[u] = (float)xs[i + u * 256];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) s = fmaf(v[u], v[u], s);
+  }
+  for (; i < cols; i += 256) {
     float v = (float)xs[i];
     s = fmaf(v, v, s);
   }
-  const float total = block256_sum_ref_order(s, red);
+  const float total = block256_sum_ref_order_dpp(s, red);
   const float rms_inv = 1.0f / sqrtf(total / (float)cols + eps);
-  if (vec) {
+  if (few) {
+#pragma unroll
+    for (int j = 0; j < P; ++j) {
+      const int i = (threadIdx.x + 256 * j) * 8;
+      if (i < cols) {
+        const half8_t xv = *reinterpret_cast<const half8_t*>(xs + i);
+        half8_t r;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const half_t inner = round_f16((float)xv[e] * rms_inv);
+          r[e] = round_f16((float)wp[j][e] * (float)inner);
+        }
+        *reinterpret_cast<half8_t*>(y + i) = r;
+      }
+    }
+  } else if (vec) {
     for (int i = threadIdx.x * 8; i < cols; i += 256 * 8) {
       const half8_t xv = *reinterpret_cast<const half8_t*>(xs + i);
       const half8_t wv = *reinterpret_cast<const half8_t*>(weights + i);

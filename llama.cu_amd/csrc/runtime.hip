@@ -40,7 +40,7 @@ workspace_t workspace_for(hipStream_t stream) {
   if (st == nullptr || !st->ready) {
     return workspace_t{};
   }
-  return workspace_t{st->workspace, st->workspace_bytes};
+  return workspace_t{st->workspace, st->workspace_bytes, st->workspace_sync};
 }
 
 device_state* current_device_state() {
@@ -77,8 +77,9 @@ int lcu_init(int device) {
   // 256 x 3 partial sums; decode attention over long rows: its scores; GEMMs with few rows: the
   // fp32 partial sums of their K splits); streams from lcu_stream_create bring their own
   st.workspace_bytes = WORKSPACE_BYTES;
-  LCU_HIP(hipMalloc(&st.workspace, st.workspace_bytes));
-  LCU_HIP(hipMemset(st.workspace, 0, st.workspace_bytes));
+  LCU_HIP(hipMalloc(&st.workspace, st.workspace_bytes + SYNC_WORDS * sizeof(uint32_t)));
+  LCU_HIP(hipMemset(st.workspace, 0, st.workspace_bytes + SYNC_WORDS * sizeof(uint32_t)));
+  st.workspace_sync = reinterpret_cast<uint32_t*>((char*)st.workspace + st.workspace_bytes);
   LCU_HIP(hipDeviceSynchronize());
   const int rc = attention_static_init(device);
   if (rc != LCU_OK) {
@@ -169,10 +170,14 @@ int lcu_stream_create(void** out_stream) {
   // graph capture, where nothing may be allocated
   workspace_t ws;
   ws.bytes = WORKSPACE_BYTES;
-  hipError_t e = hipMalloc(&ws.ptr, ws.bytes);
+  hipError_t e = hipMalloc(&ws.ptr, ws.bytes + SYNC_WORDS * sizeof(uint32_t));
   if (e == hipSuccess) {
-    e = hipMemset(ws.ptr, 0, ws.bytes);
+    e = hipMemset(ws.ptr, 0, ws.bytes + SYNC_WORDS * sizeof(uint32_t));
   }
+  if (e == hipSuccess) {
+    e = hipDeviceSynchronize();  // the clearing is done before any stream can use the flags
+  }
+  ws.sync = reinterpret_cast<uint32_t*>((char*)ws.ptr + ws.bytes);
   if (e != hipSuccess) {
     (void)hipFree(ws.ptr);
     (void)hipStreamDestroy(s);
@@ -203,6 +208,15 @@ int lcu_stream_destroy(void* stream) {
       LCU_HIP(hipFree(ws.ptr));
     }
   }
+  return LCU_OK;
+}
+
+int lcu_sync_timeouts(void* stream, unsigned* out_count) {
+  LCU_REQUIRE(out_count != nullptr, "lcu_sync_timeouts: null output");
+  const workspace_t ws = workspace_for(as_stream(stream));
+  if (ws.sync == nullptr) return set_error(LCU_E_NOINIT, "lcu_sync_timeouts: lcu_init has not run on this device");
+  LCU_HIP(hipMemcpyAsync(out_count, ws.sync + SYNC_TIMEOUTS, sizeof(unsigned), hipMemcpyDeviceToHost, as_stream(stream)));
+  LCU_HIP(hipStreamSynchronize(as_stream(stream)));
   return LCU_OK;
 }
 

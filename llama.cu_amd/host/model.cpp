@@ -338,8 +338,9 @@ void llama_context_impl::enqueue_layers(int n) {
       LCU_CHECK(lcu_decode_qkv(t_xq_.data(), kc, vc, t_norm_.data(), nullptr, L.wq.data.data(), L.wk.data.data(),
                                L.wv.data.data(), L.wq.scales.data(), L.wk.scales.data(), L.wv.scales.data(), block, dim,
                                heads, 0, t_step_.data(), p.norm_eps, rope_table_, context_len_, stream_));
-      LCU_CHECK(lcu_attention_decode(t_out_.data(), t_xq_.data(), kc, vc, t_step_.data(), decode_bound_, dim, heads,
-                                     stream_));
+      LCU_CHECK(lcu_attention_decode_spread(t_out_.data(), t_xq_.data(), kc, vc, t_step_.data(),
+                                            (char*)t_step_.data() + offsetof(step_state, seq), (int)(l & 1023),
+                                            decode_bound_, dim, heads, stream_));
     } else {
       char* k_new = kc + (size_t)sp * dim * 2;
       char* v_new = vc + (size_t)sp * dim * 2;
@@ -452,6 +453,7 @@ short llama_context_impl::next_token(std::vector<short> const& new_tokens) {
     ++samples_drawn_;
   }
   if (n == 1 || sampling_) {
+    ++host_step_.seq;
     LCU_CHECK(lcu_h2d(t_step_.data(), &host_step_, sizeof(host_step_), stream_));
   }
   if (n == 1) {

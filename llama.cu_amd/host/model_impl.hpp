@@ -81,14 +81,17 @@ struct llama_context_impl final : public llama_context {
   std::vector<kv_cache_layer> kv_;
   gpu_buffer t_embed_, t_norm_, t_xq_, t_out_, t_w1_, t_w3_, t_silu_;
   gpu_buffer t_tokens_, t_logits_, t_probs_, t_argmax_;
-  // step state on the device: {int32 position, int16 token, 64 random bits}; the decode kernels
-  // and the sampler read it from here, so one captured graph replays for every step
+  // step state on the device: {int32 position, int16 token, 64 random bits, uint32 step counter};
+  // the decode kernels and the sampler read it from here, so one captured graph replays for every
+  // step (the counter differs from step to step: the epoch of the attention kernel's hand-over)
   gpu_buffer t_step_;
   struct step_state {
     int32_t pos;
     int16_t token;
     int16_t pad;
     uint64_t random;  // this step's 64 random bits when sampling
+    uint32_t seq;     // counts the one-token steps of this context
+    uint32_t pad2;
   } host_step_{};
   bool sampling_{false};
   uint64_t sample_seed_{0};

@@ -590,6 +590,66 @@ def test_attention_decode_twice_reuses_workspace(gpu):
     G.release()
 
 
+@pytest.mark.parametrize("heads,ctx", [(32, 1024), (52, 2048), (3, 4096)])
+def test_attention_decode_spread_in_a_replayed_graph(gpu, heads, ctx):
+    """lcu_attention_decode_spread (eight workgroups per head that hand their scores over inside the launch):
+    two calls with different salts captured in one graph, replayed with the position and the step counter
+    changed on the device between replays (positions going up and down, so rows hold scores of earlier
+    epochs), every replay bit-exact against the kernel-order oracle and against lcu_attention_decode; no
+    bounded wait ran out."""
+    import ctypes as C
+    G = gpu
+    L = G.L()
+    dim = heads * 128
+    k = [normal((ctx, dim), 0, 1200 + i, 1.0) for i in range(2)]
+    v = [normal((ctx, dim), 0, 1210 + i, 1.0) for i in range(2)]
+    q = [normal((1, dim), 0, 1220 + i, 1.0) for i in range(2)]
+    kd, vd, qd = [G.dev_keep(a) for a in k], [G.dev_keep(a) for a in v], [G.dev_keep(a) for a in q]
+    out = [G.empty((1, dim)) for _ in range(2)]
+    old = G.empty((1, dim))
+    stream = C.c_void_p()
+    G.B.check(L.lcu_stream_create(C.byref(stream)))
+    state = G.B.DeviceBuffer(8)  # int32 position, uint32 step counter
+    def set_state(pos, seq):
+        a = np.array([pos, seq], dtype=np.uint32)
+        G.B.check(L.lcu_h2d(state.ptr, a.ctypes.data_as(C.c_void_p), 8, stream))
+        G.B.check(L.lcu_sync(stream))
+    def enqueue():
+        for i in range(2):
+            G.B.check(L.lcu_attention_decode_spread(out[i].ptr, qd[i].ptr, kd[i].ptr, vd[i].ptr, state.ptr, state.ptr + 4,
+                                                    i, ctx, dim, heads, stream))
+    positions = [5, ctx - 1, 300, 0, 1023 if ctx > 1023 else ctx // 2, 17, ctx - 2]
+    set_state(positions[0], 1)
+    enqueue()  # eager
+    G.B.check(L.lcu_sync(stream))
+    G.B.check(L.lcu_graph_begin_capture(stream))
+    enqueue()
+    graph = C.c_void_p()
+    G.B.check(L.lcu_graph_end_capture(stream, C.byref(graph)))
+    for step, pos in enumerate(positions):
+        set_state(pos, 2 + step)
+        G.B.check(L.lcu_graph_launch(graph, stream))
+        G.B.check(L.lcu_sync(stream))
+        T = pos + 1
+        for i in range(2):
+            got = G.host(out[i], (1, dim))
+            assert G.ulp_mismatch(got, O.attention_decode_kernel_order(q[i], k[i][:T], v[i][:T], heads)) == 0.0, (pos, i)
+            G.B.check(L.lcu_attention_decode(old.ptr, qd[i].ptr, kd[i].ptr, vd[i].ptr, state.ptr, ctx, dim, heads, stream))
+            G.B.check(L.lcu_sync(stream))
+            assert G.ulp_mismatch(got, G.host(old, (1, dim))) == 0.0, (pos, i)
+    count = C.c_uint(123)
+    G.B.check(L.lcu_sync_timeouts(stream, C.byref(count)))
+    assert count.value == 0
+    assert L.lcu_attention_decode_spread(out[0].ptr, qd[0].ptr, kd[0].ptr, vd[0].ptr, state.ptr, state.ptr + 4, 1024, ctx,
+                                         dim, heads, stream) == -2
+    assert L.lcu_attention_decode_spread(out[0].ptr, qd[0].ptr, kd[0].ptr, vd[0].ptr, state.ptr, None, 0, ctx, dim, heads,
+                                         stream) == -2
+    G.B.check(L.lcu_graph_destroy(graph))
+    G.B.check(L.lcu_stream_destroy(stream))
+    state.free()
+    G.release()
+
+
 @pytest.mark.parametrize("B,dim,heads,ffn,u8", [(8, 4096, 32, 11008, False), (8, 4096, 32, 11008, True), (33, 1024, 8, 2816, False),
                                                 (3, 320, 2, 704, False), (1, 512, 4, 1408, True)])
 def test_batch_fused_steps_equal_their_separate_operators(gpu, B, dim, heads, ffn, u8):

@@ -175,6 +175,20 @@ int lcu_attention_decode_spread(void* out_dev, const void* q_dev, const void* k_
                                 const void* pos_dev, const void* seq_dev, int salt, int max_T, int dim, int n_heads,
                                 void* stream);
 
+/* lcu_attention_decode_spread, then x += att . Wo^T (llama_cu.cu:1174, fp16 Wo [dim, dim]) and
+ * norm_out = rms_norm(x) with norm_w (1176), in one launch of one 1024-thread workgroup per compute
+ * unit: each owns 16 rows of everything, holds its rows of Wo in registers while the attention
+ * runs, and takes part in three more hand-overs like the scores' (same epoch rule, same bounded
+ * waits).  Same bits as lcu_attention_decode + lcu_gemm_f16_nt (beta 1) + lcu_rmsnorm.  max_T <= 1024;
+ * 8 * n_heads workgroups wait for one another and must all be resident, one per compute unit: more
+ * heads than a eighth of the compute units are refused (LCU_E_SHAPE), and on a device whose compute
+ * units other work holds for good the waits run out (lcu_sync_timeouts) and the result is undefined.
+ * x_io_dev: the residual row, updated in place. */
+int lcu_decode_attention_wo_norm(void* x_io_dev, void* norm_out_dev, const void* q_dev, const void* k_dev,
+                                 const void* v_dev, const void* wo_dev, const void* norm_w_dev, float eps,
+                                 const void* pos_dev, const void* seq_dev, int salt, int max_T, int dim, int n_heads,
+                                 void* stream);
+
 /* ---- one decode step of several sequences (batching is a TODO of the reference, README.md:34):
  * the GEMMs take the n_seq rows as M; these three handle what differs per sequence.  The caches
  * are given as device arrays of n_seq pointers ([positions][dim] fp16 each), positions as n_seq

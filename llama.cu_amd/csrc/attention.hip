@@ -434,6 +434,331 @@ __global__ __launch_bounds__(256) void decode_attention_spread_kernel(
   }
 }
 
+// ---- decode attention, the Wo product with the residual sum, and the RMS norm that follows, in one
+// launch (llama_cu.cu:1161-1176 for one new token, fp16 weights) ---------------------------------
+// The attention above leaves HBM idle for its whole length, the Wo product behind it streams 2 dim^2
+// bytes and then a one-workgroup norm waits for a launch of its own.  Here workgroup (head h, slice)
+// -- 1024 threads, one per compute unit -- owns the 16 rows h * 128 + slice * 16 .. + 15 of
+// everything: it computes those 16 columns of the attention output (its first four wavefronts run
+// decode_attention_spread_kernel's code), keeps its 16 rows of Wo in the registers of the other
+// twelve (requested in batches while the attention runs, so the matrix streams in behind it), and
+// after two more hand-overs of the same kind
+// ({two halves, epoch} words through memory) finishes those rows of x + Wo . att and of the
+// normalised row.  The sums keep the order of the kernels this replaces: a row of Wo is summed by
+// four wavefronts as gemv_kernel<false, 1 or 2, 2, 0> does it (chunk c of 512 elements to
+// wavefront (c / 2) % 4, two accumulators per lane, wave_sum, wavefronts in order, then
+// fmaf(1, x, sum)), the norm by 256 threads as rmsnorm_kernel.  NB: dim <= 4096 * NB.
+constexpr int FUSED_THREADS = 1024;
+constexpr int FUSED_PAD_LDS = 72 << 10;  // dynamic LDS nobody touches: a second workgroup does not fit the compute unit
+
+// offsets (in 8-byte words) of the hand-over areas behind the scores
+constexpr int EXCH_ATT = MAX_HEADS * MAX_T_DECODE;  // attention output, dim / 2 words
+constexpr int EXCH_X = EXCH_ATT + 4096;             // new residual row, dim / 2 words
+
+__device__ __forceinline__ uint4_t request_u128_device_scope(const void* p) {
+  uint4_t v;
+  asm volatile("global_load_dwordx4 %0, %1, off sc0 sc1" : "=v"(v) : "v"(p) : "memory");
+  return v;
+}
+
+// All threads of the workgroup: waits until the dim / 2 {half2, epoch} words at `words` carry this
+// launch's epoch and copies their halves to xs[0 .. dim).  Every thread asks for two words at a time.
+__device__ __forceinline__ void gather_row(half_t* xs, const uint64_t* words, int dim, uint32_t epoch,
+                                           uint32_t* timeouts) {
+  const int tid = threadIdx.x;
+  for (int w0 = tid * 2; w0 < dim / 2; w0 += FUSED_THREADS * 2) {
+    uint4_t raw;
+    int spins = 0;
+    while (true) {
+      raw = request_u128_device_scope(words + w0);
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      asm volatile("" : "+v"(raw));  // read only after the wait
+      const bool stale = raw[1] != epoch || raw[3] != epoch;
+      if (__builtin_amdgcn_ballot_w64(stale) == 0) break;
+      if (++spins > SPREAD_SPIN_LIMIT) {
+        if ((tid & 63) == 0) atomicAdd(timeouts, 1u);
+        break;
+      }
+      __builtin_amdgcn_s_sleep(1);
+    }
+    uint32_t* dst = reinterpret_cast<uint32_t*>(xs + 2 * w0);
+    dst[0] = raw[0];
+    dst[1] = raw[2];
+  }
+}
+
+// threads 0..15 hold one half each (value of row base + tid): pairs go out as {half2, epoch} words
+__device__ __forceinline__ void publish16(uint64_t* words, int base, half_t value, uint32_t epoch) {
+  const int tid = threadIdx.x;
+  const uint32_t mine = __builtin_bit_cast(unsigned short, value);
+  const uint32_t other = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)mine, 0xB1, 0xF, 0xF, true);  // lane ^ 1
+  if ((tid & 1) == 0) {
+    const uint64_t word = ((uint64_t)epoch << 32) | (other << 16) | mine;
+    __hip_atomic_store(words + (base + tid) / 2, word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+}
+
+template <int NB>
+__global__ __launch_bounds__(FUSED_THREADS) void decode_attention_wo_norm_kernel(
+    half_t* __restrict__ x_io, half_t* __restrict__ norm_out, const half_t* __restrict__ q,
+    const half_t* __restrict__ k, const half_t* __restrict__ v, const half_t* __restrict__ wo,
+    const half_t* __restrict__ norm_w, float eps, int T_cap, int dim, int n_heads, const int* __restrict__ pos_dev,
+    uint64_t* __restrict__ exch, const uint32_t* __restrict__ seq_dev, uint32_t epoch,
+    uint32_t* __restrict__ timeouts) {
+  constexpr int NJ = 4;  // rows of up to 1024 scores
+  __shared__ half_t sc[256 * NJ];
+  __shared__ float gsum[64][17];
+  __shared__ __attribute__((aligned(16))) float red[8];
+  __shared__ __attribute__((aligned(16))) half_t xs[4096 * NB];
+  __shared__ float part[16][4];
+  const int b = blockIdx.x, tid = threadIdx.x;
+  const int slice = (b >> 3) & 7, h = (b & 7) + 8 * (b >> 6);
+  if (h >= n_heads) return;
+  const int lane = tid & 63, wave = tid >> 6, team = wave >> 2, tw = wave & 3;
+  const int row0 = h * HD + slice * 16;  // first of this workgroup's 16 rows / columns
+  const bool att = tid < 256;
+  int T = T_cap;
+  if (pos_dev) T = min(max(*pos_dev + 1, 1), T_cap);
+  if (seq_dev) epoch = (epoch | (*seq_dev << 10)) & 0x7fffffffu;
+  uint64_t* srow = exch + (size_t)h * T_cap;
+
+  // ---- this workgroup's rows of Wo live in the registers of wavefronts 4-15: row team - 1 + 3 i of
+  // the 16 goes to the four wavefronts of `team` (1..3).  The requests go out in four batches, one
+  // before the attention starts and one behind each of its first three barriers, and nobody waits
+  // for them before the attention output is in: the compute unit's memory pipeline serves requests
+  // in order, so the attention's own hand-over reads only ever queue behind one batch.
+  constexpr int ROWS = 6, LOADS = ROWS * NB * 2;
+  constexpr int B0 = LOADS / 3, B1 = B0 + LOADS / 4, B2 = B1 + LOADS / 4;
+  uint4_t wreg[ROWS][NB][2];
+  auto load_wo = [&](int first, int last) {
+    if (team == 0) return;
+#pragma unroll
+    for (int i = 0; i < ROWS; ++i) {
+      const int r = min(team - 1 + 3 * i, 15);
+      const half_t* wrow = wo + (size_t)(row0 + r) * dim;
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb) {
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+          const int j = (i * NB + nb) * 2 + u;
+          if (j >= first && j < last) {
+            const int kk = min(((nb * 4 + tw) * 2 + u) * 512 + lane * 8, dim - 8);
+            wreg[i][nb][u] = __builtin_nontemporal_load(reinterpret_cast<const uint4_t*>(wrow + kk));
+          }
+        }
+      }
+    }
+  };
+  if (team > 0) __builtin_amdgcn_s_sleep(24);  // lets the attention's K and V requests go first
+  load_wo(0, B0);
+
+  // ---- attention, first part (wavefronts 0-3): scores of this slice, hand-over, row maximum
+  const int vsub = tid & 3, vg = tid >> 2;
+  half4_t vv[16];
+  float x[NJ];
+  float m = -INFINITY;
+  if (att) {
+    const int sub = tid & 15, grp = tid >> 4;
+    const half_t* kh = k + h * HD + sub * 8;
+    half8_t kv[8];
+#pragma unroll
+    for (int f = 0; f < 8; ++f) {
+      const int p = slice * 16 + grp + 128 * f;
+      kv[f] = p < T ? __builtin_nontemporal_load(reinterpret_cast<const half8_t*>(kh + (size_t)p * dim))
+                    : (half8_t)(0.0f);
+    }
+    const half8_t qh = *reinterpret_cast<const half8_t*>(q + h * HD + sub * 8);
+    const half_t* vh = v + row0 + vsub * 4;
+#pragma unroll
+    for (int f = 0; f < 16; ++f) {
+      const int p = vg + 64 * f;
+      vv[f] = p < T ? *reinterpret_cast<const half4_t*>(vh + (size_t)p * dim) : (half4_t)(0.0f);
+    }
+    const float denom = sqrtf((float)HD);
+#pragma unroll
+    for (int f = 0; f < 8; ++f) {
+      const int p = slice * 16 + grp + 128 * f;
+      float s = 0.0f;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) s = fmaf((float)qh[e], (float)kv[f][e], s);
+      s = row16_sum(s);
+      if (sub == 0 && p < T) {
+        const half_t val = round_f16(s / denom);  // 425
+        const uint64_t word = ((uint64_t)epoch << 32) | __builtin_bit_cast(unsigned short, val);
+        __hip_atomic_store(srow + p, word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+    }
+    uint64_t raw[NJ];
+    int spins = 0;
+    while (true) {
+#pragma unroll
+      for (int j = 0; j < NJ; ++j) {
+        raw[j] = tid + 256 * j < T ? request_u64_device_scope(srow + tid + 256 * j) : ((uint64_t)epoch << 32) | 0xfc00u;
+      }
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      bool stale = false;
+#pragma unroll
+      for (int j = 0; j < NJ; ++j) {
+        asm volatile("" : "+v"(raw[j]));
+        stale |= (uint32_t)(raw[j] >> 32) != epoch;
+      }
+      if (__builtin_amdgcn_ballot_w64(stale) == 0) break;
+      if (++spins > SPREAD_SPIN_LIMIT) {
+        if (lane == 0) atomicAdd(timeouts, 1u);
+        break;
+      }
+      __builtin_amdgcn_s_sleep(1);
+    }
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) x[j] = (float)__builtin_bit_cast(half_t, (unsigned short)raw[j]);
+    m = x[0];
+#pragma unroll
+    for (int j = 1; j < NJ; ++j) m = fmaxf(m, x[j]);
+    m = wave_max_dpp(m);
+    if (lane == 0) red[wave] = m;
+  }
+  __syncthreads();  // (1)
+
+  load_wo(B0, B1);
+
+  // ---- attention, second part: softmax_rows (433-499) and the weighted sum (511-531)
+  float ssum = 0.0f;
+  if (att) {
+    const float4_t r = *reinterpret_cast<const float4_t*>(red);
+    m = fmaxf(fmaxf(r[0], r[1]), fmaxf(r[2], r[3]));
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) {
+      if (tid + 256 * j < T) {
+        x[j] = exp_ieee(x[j] - m);
+        ssum += x[j];
+      }
+    }
+    ssum += __shfl_xor(ssum, 16, WAVE);
+    ssum += dpp_f32<0x128>(ssum);
+    {
+      const int vi = __builtin_bit_cast(int, ssum);
+      int t = __builtin_amdgcn_update_dpp(0, vi, 0x104, 0xF, 0x5, false);
+      t = __builtin_amdgcn_update_dpp(t, vi, 0x114, 0xF, 0xA, false);
+      ssum += __builtin_bit_cast(float, t);
+    }
+    ssum += dpp_f32<0x4E>(ssum);
+    ssum += dpp_f32<0xB1>(ssum);
+  }
+  __syncthreads();  // (2) every attention wavefront has read the maxima
+  load_wo(B1, B2);
+  if (att && (tid & 31) == 0) red[tid >> 5] = ssum;
+  __syncthreads();  // (3)
+  load_wo(B2, LOADS);
+  if (att) {
+    const float4_t lo = *reinterpret_cast<const float4_t*>(red), hi = *reinterpret_cast<const float4_t*>(red + 4);
+    const float total = ((lo[0] + hi[0]) + (lo[2] + hi[2])) + ((lo[1] + hi[1]) + (lo[3] + hi[3]));
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) {
+      if (tid + 256 * j < T) sc[tid + 256 * j] = round_f16(x[j] / total);  // 497
+    }
+  }
+  __syncthreads();  // (4)
+  if (att) {
+    float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+    for (int f = 0; f < 16; ++f) {
+      const int p = vg + 64 * f;
+      if (p < T) {
+        const float prob = (float)sc[p];
+#pragma unroll
+        for (int c = 0; c < 4; ++c) acc[c] = fmaf(prob, (float)vv[f][c], acc[c]);
+      }
+    }
+#pragma unroll
+    for (int c = 0; c < 4; ++c) gsum[vg][vsub * 4 + c] = acc[c];
+  }
+  __syncthreads();  // (5)
+  if (tid < 16) {
+    float o = 0.0f;
+#pragma unroll
+    for (int g = 0; g < 64; ++g) o += gsum[g][tid];
+    publish16(exch + EXCH_ATT, row0, round_f16(o), epoch);  // 529
+  }
+
+  // ---- x + Wo . att for the 16 rows (llama_cu.cu:1174)
+  gather_row(xs, exch + EXCH_ATT, dim, epoch, timeouts);
+  __syncthreads();  // (6)
+  if (team > 0) {
+    half8_t xp[NB][2];  // this lane's pieces of the attention output, the same for every row
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) {
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {
+        const int kk = min(((nb * 4 + tw) * 2 + u) * 512 + lane * 8, dim - 8);
+        xp[nb][u] = *reinterpret_cast<const half8_t*>(xs + kk);
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < ROWS; ++i) {
+      const int r = team - 1 + 3 * i;
+      float a0 = 0.0f, a1 = 0.0f;
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb) {
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+          const int kk = ((nb * 4 + tw) * 2 + u) * 512 + lane * 8;
+          if (kk < dim) {
+            const half8_t xv = xp[nb][u];
+            const half8_t wv = __builtin_bit_cast(half8_t, wreg[i][nb][u]);
+#pragma unroll
+            for (int e = 0; e < 8; e += 2) {
+              a0 = fmaf((float)wv[e], (float)xv[e], a0);
+              a1 = fmaf((float)wv[e + 1], (float)xv[e + 1], a1);
+            }
+          }
+        }
+      }
+      const float s = wave_sum(a0 + a1);
+      if (lane == 0 && r < 16) part[r][tw] = s;
+    }
+  }
+  __syncthreads();  // (7) also: every read of the attention output in xs is done
+  if (tid < 16) {
+    float acc = 0.0f;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) acc += part[tid][w];
+    const half_t xn = round_f16(fmaf(1.0f, (float)x_io[row0 + tid], acc));  // llama_cu.cu:279 with beta = 1
+    x_io[row0 + tid] = xn;
+    publish16(exch + EXCH_X, row0, xn, epoch);
+  }
+
+  // ---- rms_norm of the new row (llama_cu.cu:1176, 66-107): every workgroup sums the squares, each
+  // normalises its own 16 elements
+  gather_row(xs, exch + EXCH_X, dim, epoch, timeouts);
+  __syncthreads();  // (8)
+  float sq = 0.0f;
+  if (att) {
+    for (int i = tid; i < dim; i += 256) {
+      const float e = (float)xs[i];
+      sq = fmaf(e, e, sq);
+    }
+    sq += __shfl_xor(sq, 16, WAVE);
+    sq += dpp_f32<0x128>(sq);
+    {
+      const int vi = __builtin_bit_cast(int, sq);
+      int t = __builtin_amdgcn_update_dpp(0, vi, 0x104, 0xF, 0x5, false);
+      t = __builtin_amdgcn_update_dpp(t, vi, 0x114, 0xF, 0xA, false);
+      sq += __builtin_bit_cast(float, t);
+    }
+    sq += dpp_f32<0x4E>(sq);
+    sq += dpp_f32<0xB1>(sq);
+    if ((tid & 31) == 0) red[tid >> 5] = sq;
+  }
+  __syncthreads();  // (9)
+  if (tid < 16) {
+    const float4_t lo = *reinterpret_cast<const float4_t*>(red), hi = *reinterpret_cast<const float4_t*>(red + 4);
+    const float total = ((lo[0] + hi[0]) + (lo[2] + hi[2])) + ((lo[1] + hi[1]) + (lo[3] + hi[3]));
+    const float rms_inv = 1.0f / sqrtf(total / (float)dim + eps);
+    const half_t inner = round_f16((float)xs[row0 + tid] * rms_inv);
+    norm_out[row0 + tid] = round_f16((float)norm_w[row0 + tid] * (float)inner);
+  }
+}
+
 // seq_dev == nullptr: the epoch is a number the host draws per launch (never under stream capture:
 // a replay would repeat it); else it comes from *seq_dev, which the caller changes before every
 // run, and `salt`.  The score words live in the exchange area behind the stream's workspace.
@@ -811,6 +1136,55 @@ int lcu_attention_decode_spread(void* out_dev, const void* q_dev, const void* k_
   return launch_decode_attention_spread((half_t*)out_dev, (const half_t*)q_dev, (const half_t*)k_dev,
                                         (const half_t*)v_dev, (const int*)pos_dev, max_T, dim, n_heads, ws,
                                         (const uint32_t*)seq_dev, (uint32_t)salt, as_stream(stream));
+}
+
+int lcu_decode_attention_wo_norm(void* x_io_dev, void* norm_out_dev, const void* q_dev, const void* k_dev,
+                                 const void* v_dev, const void* wo_dev, const void* norm_w_dev, float eps,
+                                 const void* pos_dev, const void* seq_dev, int salt, int max_T, int dim, int n_heads,
+                                 void* stream) {
+  LCU_REQUIRE(x_io_dev && norm_out_dev && q_dev && k_dev && v_dev && wo_dev && norm_w_dev && pos_dev && seq_dev,
+              "lcu_decode_attention_wo_norm: null pointer");
+  LCU_REQUIRE(n_heads > 0 && n_heads <= MAX_HEADS && dim == n_heads * HD,
+              "lcu_decode_attention_wo_norm: dim %d / heads %d unsupported (head_dim must be 128, at most %d heads)",
+              dim, n_heads, MAX_HEADS);
+  LCU_REQUIRE(max_T > 0 && max_T <= 1024, "lcu_decode_attention_wo_norm: max_T %d outside 1..1024", max_T);
+  LCU_REQUIRE(salt >= 0 && salt < 1024, "lcu_decode_attention_wo_norm: salt %d outside 0..1023", salt);
+  const workspace_t ws = workspace_for(as_stream(stream));
+  if (ws.sync == nullptr) {
+    return set_error(LCU_E_NOINIT, "lcu_decode_attention_wo_norm: lcu_init has not run on this device");
+  }
+  // the workgroups wait for one another, so all of them must be resident at once: one per compute unit
+  device_state* ds = current_device_state();
+  LCU_REQUIRE(ds != nullptr && n_heads * SPREAD <= ds->compute_units,
+              "lcu_decode_attention_wo_norm: %d heads need %d compute units", n_heads, n_heads * SPREAD);
+  static_assert(SYNC_WORDS - SYNC_EXCHANGE >= (EXCH_X + 4096) * 2, "exchange area");
+  static_assert(MAX_HEADS * HD / 2 <= 4096, "hand-over areas hold dim / 2 words");
+  uint64_t* exch = reinterpret_cast<uint64_t*>(ws.sync + SYNC_EXCHANGE);
+  const int grid = (n_heads + 7) / 8 * 8 * SPREAD;
+  hipStream_t s = as_stream(stream);
+  static bool attr_set[16] = {};
+  int dev = 0;
+  LCU_HIP(hipGetDevice(&dev));
+  if (!attr_set[dev & 15]) {
+    LCU_HIP(hipFuncSetAttribute((const void*)decode_attention_wo_norm_kernel<1>,
+                                hipFuncAttributeMaxDynamicSharedMemorySize, FUSED_PAD_LDS));
+    LCU_HIP(hipFuncSetAttribute((const void*)decode_attention_wo_norm_kernel<2>,
+                                hipFuncAttributeMaxDynamicSharedMemorySize, FUSED_PAD_LDS));
+    attr_set[dev & 15] = true;
+  }
+  if (dim <= 4096) {
+    decode_attention_wo_norm_kernel<1><<<grid, FUSED_THREADS, FUSED_PAD_LDS, s>>>(
+        (half_t*)x_io_dev, (half_t*)norm_out_dev, (const half_t*)q_dev, (const half_t*)k_dev, (const half_t*)v_dev,
+        (const half_t*)wo_dev, (const half_t*)norm_w_dev, eps, max_T, dim, n_heads, (const int*)pos_dev, exch,
+        (const uint32_t*)seq_dev, (uint32_t)salt, ws.sync + SYNC_TIMEOUTS);
+  } else {
+    decode_attention_wo_norm_kernel<2><<<grid, FUSED_THREADS, FUSED_PAD_LDS, s>>>(
+        (half_t*)x_io_dev, (half_t*)norm_out_dev, (const half_t*)q_dev, (const half_t*)k_dev, (const half_t*)v_dev,
+        (const half_t*)wo_dev, (const half_t*)norm_w_dev, eps, max_T, dim, n_heads, (const int*)pos_dev, exch,
+        (const uint32_t*)seq_dev, (uint32_t)salt, ws.sync + SYNC_TIMEOUTS);
+  }
+  LCU_LAUNCH_CHECK();
+  return LCU_OK;
 }
 
 int lcu_attention_decode_static(void* out_dev, const void* q_dev, const void* k_dev, const void* v_dev, int T, int dim,

@@ -235,6 +235,9 @@ llama_context_impl::llama_context_impl(llama_model* model, int context_len, floa
     : llama_context(static_cast<llama_model_impl*>(model), context_len, temperature) {
   LCU_CHECK(lcu_init(0));
   LCU_CHECK(lcu_stream_create(&stream_));
+  lcu_device_props props;
+  LCU_CHECK(lcu_device_get_props(0, &props));
+  compute_units_ = props.compute_units;
   const int head_dim = model_->params.dim / model_->params.n_heads;
   LCU_CHECK(lcu_rope_table_create(&rope_table_, context_len_, head_dim, 10000.0f));  // theta: llama_cu.cu:374
   clear_tokens();
@@ -332,15 +335,25 @@ void llama_context_impl::enqueue_layers(int n) {
     llama_layer const& L = model_->layers[l];
     char* kc = (char*)kv_[l].k.data();
     char* vc = (char*)kv_[l].v.data();
+    bool fused_wo = false;
     if (n == 1) {
       // 1129, then 1144-1156 in one launch, then 1161-1171 in one launch
       LCU_CHECK(lcu_rmsnorm(t_norm_.data(), x, L.attn_norm.data(), 1, dim, p.norm_eps, stream_));
       LCU_CHECK(lcu_decode_qkv(t_xq_.data(), kc, vc, t_norm_.data(), nullptr, L.wq.data.data(), L.wk.data.data(),
                                L.wv.data.data(), L.wq.scales.data(), L.wk.scales.data(), L.wv.scales.data(), block, dim,
                                heads, 0, t_step_.data(), p.norm_eps, rope_table_, context_len_, stream_));
-      LCU_CHECK(lcu_attention_decode_spread(t_out_.data(), t_xq_.data(), kc, vc, t_step_.data(),
-                                            (char*)t_step_.data() + offsetof(step_state, seq), (int)(l & 1023),
-                                            decode_bound_, dim, heads, stream_));
+      const void* seq = (char*)t_step_.data() + offsetof(step_state, seq);
+      // fp16 weights and rows of up to 1024 scores: attention, the Wo product with the residual sum
+      // (1174) and the norm that follows (1176) in one launch
+      fused_wo = !L.wo.quantised && decode_bound_ <= 1024 && heads * 8 <= compute_units_;
+      if (fused_wo) {
+        LCU_CHECK(lcu_decode_attention_wo_norm(x, t_norm_.data(), t_xq_.data(), kc, vc, L.wo.data.data(),
+                                               L.ffn_norm.data(), p.norm_eps, t_step_.data(), seq, (int)(l & 1023),
+                                               decode_bound_, dim, heads, stream_));
+      } else {
+        LCU_CHECK(lcu_attention_decode_spread(t_out_.data(), t_xq_.data(), kc, vc, t_step_.data(), seq,
+                                              (int)(l & 1023), decode_bound_, dim, heads, stream_));
+      }
     } else {
       char* k_new = kc + (size_t)sp * dim * 2;
       char* v_new = vc + (size_t)sp * dim * 2;
@@ -352,8 +365,10 @@ void llama_context_impl::enqueue_layers(int n) {
       LCU_CHECK(lcu_rope(k_new, k_new, n, dim, heads, sp, rope_table_, context_len_, stream_));  // 1152, new rows only
       LCU_CHECK(lcu_attention(t_out_.data(), t_xq_.data(), kc, vc, n, T, sp, dim, heads, stream_));          // 1161-1171
     }
-    matmul(x, t_out_.data(), L.wo, n, 1.0f);                                                                 // 1174
-    LCU_CHECK(lcu_rmsnorm(t_norm_.data(), x, L.ffn_norm.data(), n, dim, p.norm_eps, stream_));               // 1176
+    if (!fused_wo) {
+      matmul(x, t_out_.data(), L.wo, n, 1.0f);                                                               // 1174
+      LCU_CHECK(lcu_rmsnorm(t_norm_.data(), x, L.ffn_norm.data(), n, dim, p.norm_eps, stream_));             // 1176
+    }
     if (n == 1) {
       // 1180-1183 in one launch
       LCU_CHECK(lcu_decode_ffn_up(t_silu_.data(), t_norm_.data(), nullptr, L.w1.data.data(), L.w3.data.data(),

@@ -99,6 +99,7 @@ struct llama_context_impl final : public llama_context {
   void* decode_graph_{nullptr};
   int decode_calls_{0};
   int decode_bound_{0};  // the position bound the decode graph was captured with
+  int compute_units_{0};
   void* stream_{nullptr};
   void* rope_table_{nullptr};
   int last_n_{0};

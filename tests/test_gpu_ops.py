@@ -650,6 +650,74 @@ def test_attention_decode_spread_in_a_replayed_graph(gpu, heads, ctx):
     G.release()
 
 
+@pytest.mark.parametrize("heads,ctx", [(32, 1024), (8, 640), (3, 1024), (24, 300)])
+def test_decode_attention_wo_norm_equals_its_separate_operators(gpu, heads, ctx):
+    """lcu_decode_attention_wo_norm (attention, x += att . Wo^T and the RMS norm behind it in one launch with
+    in-launch hand-overs) against lcu_attention_decode + lcu_gemm_f16_nt (beta 1) + lcu_rmsnorm and against the
+    kernel-order oracle, bit for bit: eager, captured and replayed with positions going up and down."""
+    import ctypes as C
+    G = gpu
+    L = G.L()
+    dim = heads * 128
+    eps = 1e-5
+    k, v = normal((ctx, dim), 0, 1300, 1.0), normal((ctx, dim), 0, 1301, 1.0)
+    q, x0 = normal((1, dim), 0, 1302, 1.0), normal((1, dim), 0, 1303, 1.0)
+    wo, nw = normal((dim, dim), 0, 1304, 0.02), normal((dim,), 1, 1305, 0.1)
+    kd, vd, qd, wod, nwd = [G.dev_keep(a) for a in (k, v, q, wo, nw)]
+    x_f, n_f = G.empty((1, dim)), G.empty((1, dim))       # fused
+    x_s, n_s, att_s = G.empty((1, dim)), G.empty((1, dim)), G.empty((1, dim))  # separate
+    stream = C.c_void_p()
+    G.B.check(L.lcu_stream_create(C.byref(stream)))
+    state = G.B.DeviceBuffer(8)
+    def set_state(pos, seq):
+        a = np.array([pos, seq], dtype=np.uint32)
+        G.B.check(L.lcu_h2d(state.ptr, a.ctypes.data_as(C.c_void_p), 8, stream))
+        for dst in (x_f, x_s):
+            G.B.check(L.lcu_h2d(dst.ptr, x0.ctypes.data_as(C.c_void_p), x0.nbytes, stream))
+        G.B.check(L.lcu_sync(stream))
+    def fused():
+        G.B.check(L.lcu_decode_attention_wo_norm(x_f.ptr, n_f.ptr, qd.ptr, kd.ptr, vd.ptr, wod.ptr, nwd.ptr, eps, state.ptr,
+                                                 state.ptr + 4, 7, ctx, dim, heads, stream))
+    def check(pos):
+        G.B.check(L.lcu_attention_decode(att_s.ptr, qd.ptr, kd.ptr, vd.ptr, state.ptr, ctx, dim, heads, stream))
+        G.B.check(L.lcu_gemm_f16_nt(x_s.ptr, att_s.ptr, wod.ptr, 1, dim, dim, 1.0, stream))
+        G.B.check(L.lcu_rmsnorm(n_s.ptr, x_s.ptr, nwd.ptr, 1, dim, eps, stream))
+        G.B.check(L.lcu_sync(stream))
+        got_x, got_n = G.host(x_f, (1, dim)), G.host(n_f, (1, dim))
+        assert G.ulp_mismatch(got_x, G.host(x_s, (1, dim))) == 0.0, pos
+        assert G.ulp_mismatch(got_n, G.host(n_s, (1, dim))) == 0.0, pos
+        T = pos + 1
+        att = O.attention_decode_kernel_order(q, k[:T], v[:T], heads)
+        want_x = O.matmul_nt(att, wo, flavour=2, beta=1.0, out=x0)
+        assert G.ulp_mismatch(got_x, want_x) == 0.0, pos
+        assert G.ulp_mismatch(got_n, O.rms_norm(want_x, nw, eps)) == 0.0, pos
+    positions = [4, ctx - 1, 200, 0, ctx // 2, ctx - 2]
+    set_state(positions[0], 1)
+    fused()
+    check(positions[0])
+    set_state(positions[0], 2)
+    G.B.check(L.lcu_graph_begin_capture(stream))
+    fused()
+    graph = C.c_void_p()
+    G.B.check(L.lcu_graph_end_capture(stream, C.byref(graph)))
+    for step, pos in enumerate(positions):
+        set_state(pos, 3 + step)
+        G.B.check(L.lcu_graph_launch(graph, stream))
+        check(pos)
+    count = C.c_uint(123)
+    G.B.check(L.lcu_sync_timeouts(stream, C.byref(count)))
+    assert count.value == 0
+    assert L.lcu_decode_attention_wo_norm(x_f.ptr, n_f.ptr, qd.ptr, kd.ptr, vd.ptr, wod.ptr, nwd.ptr, eps, state.ptr,
+                                          state.ptr + 4, 7, 1025, dim, heads, stream) == -2
+    # more workgroups than compute units could not all be resident while they wait for one another
+    assert L.lcu_decode_attention_wo_norm(x_f.ptr, n_f.ptr, qd.ptr, kd.ptr, vd.ptr, wod.ptr, nwd.ptr, eps, state.ptr,
+                                          state.ptr + 4, 7, ctx, 52 * 128, 52, stream) == -2
+    G.B.check(L.lcu_graph_destroy(graph))
+    G.B.check(L.lcu_stream_destroy(stream))
+    state.free()
+    G.release()
+
+
 @pytest.mark.parametrize("B,dim,heads,ffn,u8", [(8, 4096, 32, 11008, False), (8, 4096, 32, 11008, True), (33, 1024, 8, 2816, False),
                                                 (3, 320, 2, 704, False), (1, 512, 4, 1408, True)])
 def test_batch_fused_steps_equal_their_separate_operators(gpu, B, dim, heads, ffn, u8):

@@ -246,6 +246,15 @@ int lcu_decode_qkv(void* q_out_dev, void* k_cache_dev, void* v_cache_dev, const 
                    const void* sq_dev, const void* sk_dev, const void* sv_dev, int block, int dim,
                    int n_heads, int pos, const void* pos_dev, float eps, const void* rope_table_dev,
                    int table_positions, void* stream);
+/* x += lhs [1, K] . W^T (W [N, K], fp16 or uint8 codes with scales; llama_cu.cu:1185) and then
+ * norm_out = rms_norm(x) with norm_w (1129 of the next layer), in one launch: one more workgroup
+ * than the GEMV has waits inside the launch for the rows of the new x, which reach it as
+ * {two halves, epoch} words through the stream's workspace, and writes x and its norm.  The epoch is
+ * *seq_dev << 10 | salt, as for lcu_attention_decode_spread (same rule, same bounded wait).  Same
+ * bits as lcu_gemm_f16_nt / lcu_gemm_f16u8_nt (beta 1) + lcu_rmsnorm.  N <= 8192. */
+int lcu_decode_proj_norm(void* x_io_dev, void* norm_out_dev, const void* lhs_dev, const void* w_dev,
+                         const void* scales_dev, int block, int K, int N, const void* norm_w_dev, float eps,
+                         const void* seq_dev, int salt, void* stream);
 /* rms_norm(x, ffn_norm) -> W1 and W3 GEMV -> silu(w1) * w3: llama_cu.cu:1176-1183 */
 int lcu_decode_ffn_up(void* out_dev, const void* x_dev, const void* norm_w_dev, const void* w1_dev,
                       const void* w3_dev, const void* s1_dev, const void* s3_dev, int block, int dim,

@@ -451,9 +451,7 @@ __global__ __launch_bounds__(256) void decode_attention_spread_kernel(
 constexpr int FUSED_THREADS = 1024;
 constexpr int FUSED_PAD_LDS = 72 << 10;  // dynamic LDS nobody touches: a second workgroup does not fit the compute unit
 
-// offsets (in 8-byte words) of the hand-over areas behind the scores
-constexpr int EXCH_ATT = MAX_HEADS * MAX_T_DECODE;  // attention output, dim / 2 words
-constexpr int EXCH_X = EXCH_ATT + 4096;             // new residual row, dim / 2 words
+static_assert(EXCH_ATT == MAX_HEADS * MAX_T_DECODE, "the scores' area");
 
 __device__ __forceinline__ uint4_t request_u128_device_scope(const void* p) {
   uint4_t v;

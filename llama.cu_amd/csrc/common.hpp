@@ -60,12 +60,18 @@ struct workspace_t {
   // SYNC_WORDS zero-initialised uint32 behind the scratch, never used as scratch: what workgroups
   // of one launch hand to one another (decode attention spread over several workgroups per head).
   // Words 0 .. SYNC_TIMEOUTS are counters; from SYNC_EXCHANGE on, 8-byte {value, epoch} words (64
-  // heads x 4096 scores, then two rows of 4096), which no other operator may write: a reader trusts
+  // heads x 4096 scores, then three rows of 4096), which no other operator may write: a reader trusts
   // a word by its epoch.
   uint32_t* sync = nullptr;
 };
 constexpr int SYNC_EXCHANGE = 2048;
-constexpr int SYNC_WORDS = SYNC_EXCHANGE + (64 * 4096 + 2 * 4096) * 2;
+// offsets (in 8-byte words) of the hand-over areas: decode attention scores (64 heads x 4096), then
+// three rows of up to 8192 halves as {half2, epoch} words: the attention output, the residual row
+// behind Wo, the residual row behind W2
+constexpr int EXCH_ATT = 64 * 4096;
+constexpr int EXCH_X = EXCH_ATT + 4096;
+constexpr int EXCH_PROJ = EXCH_X + 4096;
+constexpr int SYNC_WORDS = SYNC_EXCHANGE + (EXCH_PROJ + 4096) * 2;
 constexpr int SYNC_TIMEOUTS = SYNC_EXCHANGE - 1;  // word that counts bounded waits which ran out
 workspace_t workspace_for(hipStream_t stream);
 

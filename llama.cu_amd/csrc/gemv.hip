@@ -335,6 +335,41 @@ struct plain_tasks {
   }
 };
 
+// rows of a product whose result is added to the residual row and then normalised (W2 of one layer,
+// the attention norm of the next: llama_cu.cu:1185, 1129): x[n] = fp16(dot + x[n]) leaves as a
+// {two halves, epoch} word for the workgroup that normalises the row (decode_proj_norm_kernel)
+template <bool U8, int R>
+struct proj_norm_tasks {
+  const void* W;
+  const half_t* S;
+  const half_t* x_old;
+  uint64_t* words;
+  int K, N, nblk;
+  uint32_t epoch;
+  __device__ __forceinline__ void rows(int task, const uint8_t* (&rows)[R], const half_t* (&srow)[R]) const {
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      const int n = min(task * R + r, N - 1);
+      rows[r] = row_ptr<U8>(W, n, K);
+      srow[r] = U8 ? S + (size_t)n * nblk : nullptr;
+    }
+  }
+  __device__ __forceinline__ void finish(int task, const float (&acc)[R]) const {
+    static_assert(R % 2 == 0, "pairs of rows");
+#pragma unroll
+    for (int r = 0; r < R; r += 2) {
+      const int n = task * R + r;
+      if (n < N) {  // N is even
+        const half_t h0 = round_f16(fmaf(1.0f, (float)x_old[n], acc[r]));          // llama_cu.cu:279 with beta = 1
+        const half_t h1 = round_f16(fmaf(1.0f, (float)x_old[n + 1], acc[r + 1]));
+        const uint64_t word = ((uint64_t)epoch << 32) | ((uint32_t)__builtin_bit_cast(unsigned short, h1) << 16) |
+                              __builtin_bit_cast(unsigned short, h0);
+        __hip_atomic_store(words + n / 2, word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+    }
+  }
+};
+
 // One of Wq / Wk / Wv (chosen per workgroup by the kernel): a task is PAIRS interleaved pairs (rows
 // 2p, 2p+1) of that matrix; RoPE on q and k (llama_cu.cu:381-387), results to q_out / the caches'
 // row for this position
@@ -500,6 +535,94 @@ __global__ __launch_bounds__(GEMV_THREADS) void decode_ffn_up_kernel(
   st.run(xs, rms_inv, part);
 }
 
+// x += lhs . W^T followed by norm_out = rms_norm(x) in one launch.  Workgroups 0 .. n_tasks - 1 are
+// the GEMV of gemv_kernel (R rows each, same sums); each hands its rows of the new x over as
+// {two halves, epoch} words written through to memory.  One more workgroup, the last of the grid,
+// asks for the N / 2 words until all of them carry this launch's epoch (a value no earlier launch
+// left there: step counter << 10 | salt), then writes the row and its norm (rmsnorm_kernel's
+// arithmetic).  It is resident while the last GEMV workgroups run, so the norm costs the hand-over
+// and its own arithmetic instead of a launch; its wait is bounded and counts itself when it runs out.
+constexpr int FOLLOW_SPIN_LIMIT = 1 << 16;
+constexpr int FOLLOW_PIECES = 8;  // 16-byte requests per thread: N <= 8192
+
+template <bool U8, int R, int U>
+__global__ __launch_bounds__(GEMV_THREADS) void decode_proj_norm_kernel(
+    half_t* __restrict__ x_io, half_t* __restrict__ norm_out, const half_t* __restrict__ lhs,
+    const void* __restrict__ W, const half_t* __restrict__ S, const half_t* __restrict__ norm_w, int K, int N, int block,
+    float eps, uint64_t* __restrict__ words, const uint32_t* __restrict__ seq_dev, uint32_t epoch,
+    uint32_t* __restrict__ timeouts) {
+  extern __shared__ half_t xs[];  // N halves: the follower's copy of the row
+  __shared__ __attribute__((aligned(16))) float red[8];
+  __shared__ float part[GEMV_WAVES * R];
+  epoch = (epoch | (*seq_dev << 10)) & 0x7fffffffu;
+  const int n_tasks = (N + R - 1) / R;
+  if ((int)blockIdx.x < n_tasks) {
+    proj_norm_tasks<U8, R> tk{W, S, x_io, words, K, N, U8 ? K / block : 0, epoch};
+    stream_t<U8, R, U, false, proj_norm_tasks<U8, R>> st(tk, lhs, nullptr, K, block, blockIdx.x);
+    st.begin();
+    st.run(xs, 1.0f, part);
+    return;
+  }
+  const int tid = threadIdx.x;
+  uint4_t raw[FOLLOW_PIECES];
+  int spins = 0;
+  while (true) {
+#pragma unroll
+    for (int j = 0; j < FOLLOW_PIECES; ++j) {
+      const int w0 = (tid + GEMV_THREADS * j) * 2;
+      if (w0 < N / 2) {
+        asm volatile("global_load_dwordx4 %0, %1, off sc0 sc1" : "=v"(raw[j]) : "v"(words + w0) : "memory");
+      }
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    bool stale = false;
+#pragma unroll
+    for (int j = 0; j < FOLLOW_PIECES; ++j) {
+      const int w0 = (tid + GEMV_THREADS * j) * 2;
+      if (w0 < N / 2) {
+        asm volatile("" : "+v"(raw[j]));  // read only after the wait
+        stale |= raw[j][1] != epoch || raw[j][3] != epoch;
+      }
+    }
+    if (__builtin_amdgcn_ballot_w64(stale) == 0) break;
+    if (++spins > FOLLOW_SPIN_LIMIT) {
+      if ((tid & 63) == 0) atomicAdd(timeouts, 1u);
+      break;
+    }
+    __builtin_amdgcn_s_sleep(8);
+  }
+#pragma unroll
+  for (int j = 0; j < FOLLOW_PIECES; ++j) {
+    const int w0 = (tid + GEMV_THREADS * j) * 2;
+    if (w0 < N / 2) {
+      uint32_t* dst = reinterpret_cast<uint32_t*>(xs + 2 * w0);
+      dst[0] = raw[j][0];
+      dst[1] = raw[j][2];
+    }
+  }
+  __syncthreads();
+  // rms_norm, llama_cu.cu:66-107, as rmsnorm_kernel: thread t owns elements t, t + 256, ...
+  float s = 0.0f;
+  for (int i = tid; i < N; i += GEMV_THREADS) {
+    const float e = (float)xs[i];
+    s = fmaf(e, e, s);
+  }
+  const float total = block256_sum_ref_order_dpp(s, red);
+  const float rms_inv = 1.0f / sqrtf(total / (float)N + eps);
+  for (int i = tid * 8; i < N; i += GEMV_THREADS * 8) {
+    const half8_t xv = *reinterpret_cast<const half8_t*>(xs + i);
+    const half8_t wv = *reinterpret_cast<const half8_t*>(norm_w + i);
+    half8_t r;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const half_t inner = round_f16((float)xv[e] * rms_inv);
+      r[e] = round_f16((float)wv[e] * (float)inner);
+    }
+    *reinterpret_cast<half8_t*>(x_io + i) = xv;
+    *reinterpret_cast<half8_t*>(norm_out + i) = r;
+  }
+}
+
 // calls f with the number of 16-byte pieces of x per thread (x_stage_t) that covers dim <= 24576
 template <class F>
 void with_x_pieces(int dim, F&& f) {
@@ -603,6 +726,41 @@ int lcu_decode_qkv(void* q_out_dev, void* k_cache_dev, void* v_cache_dev, const 
           (half_t*)q_out_dev, k_row, v_row, (const half_t*)x_dev, nullptr, wq_dev, wk_dev, wv_dev, nullptr, nullptr,
           nullptr, 0, dim, head_dim, eps, rope_row, (const int*)pos_dev, table_positions - 1);
     }
+  }
+  LCU_LAUNCH_CHECK();
+  return LCU_OK;
+}
+
+int lcu_decode_proj_norm(void* x_io_dev, void* norm_out_dev, const void* lhs_dev, const void* w_dev,
+                         const void* scales_dev, int block, int K, int N, const void* norm_w_dev, float eps,
+                         const void* seq_dev, int salt, void* stream) {
+  LCU_REQUIRE(x_io_dev && norm_out_dev && lhs_dev && w_dev && norm_w_dev && seq_dev, "lcu_decode_proj_norm: null pointer");
+  LCU_REQUIRE(K > 0 && K % 16 == 0 && N > 0 && N % 8 == 0 && N <= 2048 * FOLLOW_PIECES / 2,
+              "lcu_decode_proj_norm: bad shape K %d N %d (N a multiple of 8, at most %d)", K, N, 2048 * FOLLOW_PIECES / 2);
+  LCU_REQUIRE(salt >= 0 && salt < 1024, "lcu_decode_proj_norm: salt %d outside 0..1023", salt);
+  hipStream_t st = as_stream(stream);
+  const workspace_t ws = workspace_for(st);
+  if (ws.sync == nullptr) return set_error(LCU_E_NOINIT, "lcu_decode_proj_norm: lcu_init has not run on this device");
+  uint64_t* words = reinterpret_cast<uint64_t*>(ws.sync + SYNC_EXCHANGE) + EXCH_PROJ;
+  uint32_t* timeouts = ws.sync + SYNC_TIMEOUTS;
+  const size_t lds = (size_t)N * 2;
+  if (block > 0) {
+    int rc = check_quant_args("lcu_decode_proj_norm", scales_dev, K, block);
+    if (rc) return rc;
+    // rows per workgroup as gemv_u8 picks them
+    if (N >= 6144) {
+      decode_proj_norm_kernel<true, 4, 1><<<(N + 3) / 4 + 1, GEMV_THREADS, lds, st>>>(
+          (half_t*)x_io_dev, (half_t*)norm_out_dev, (const half_t*)lhs_dev, w_dev, (const half_t*)scales_dev,
+          (const half_t*)norm_w_dev, K, N, block, eps, words, (const uint32_t*)seq_dev, (uint32_t)salt, timeouts);
+    } else {
+      decode_proj_norm_kernel<true, 2, 1><<<(N + 1) / 2 + 1, GEMV_THREADS, lds, st>>>(
+          (half_t*)x_io_dev, (half_t*)norm_out_dev, (const half_t*)lhs_dev, w_dev, (const half_t*)scales_dev,
+          (const half_t*)norm_w_dev, K, N, block, eps, words, (const uint32_t*)seq_dev, (uint32_t)salt, timeouts);
+    }
+  } else {
+    decode_proj_norm_kernel<false, 2, 2><<<(N + 1) / 2 + 1, GEMV_THREADS, lds, st>>>(
+        (half_t*)x_io_dev, (half_t*)norm_out_dev, (const half_t*)lhs_dev, w_dev, nullptr, (const half_t*)norm_w_dev, K, N,
+        0, eps, words, (const uint32_t*)seq_dev, (uint32_t)salt, timeouts);
   }
   LCU_LAUNCH_CHECK();
   return LCU_OK;

@@ -331,14 +331,19 @@ void llama_context_impl::enqueue_layers(int n) {
   const int sp = start_pos_, T = sp + n;
   const int block = p.q_type == quantization_type::uint8 ? p.quantization_block_size : 0;
   char* x = (char*)t_embed_.data();
+  bool norm_ready = false;  // t_norm_ already holds this layer's normalised input
   for (size_t l = 0; l < model_->layers.size(); ++l) {
     llama_layer const& L = model_->layers[l];
     char* kc = (char*)kv_[l].k.data();
     char* vc = (char*)kv_[l].v.data();
     bool fused_wo = false;
     if (n == 1) {
-      // 1129, then 1144-1156 in one launch, then 1161-1171 in one launch
-      LCU_CHECK(lcu_rmsnorm(t_norm_.data(), x, L.attn_norm.data(), 1, dim, p.norm_eps, stream_));
+      // 1129 (unless the previous layer's W2 launch has left the normalised row behind), then
+      // 1144-1156 in one launch, then 1161-1171 in one launch
+      if (!norm_ready) {
+        LCU_CHECK(lcu_rmsnorm(t_norm_.data(), x, L.attn_norm.data(), 1, dim, p.norm_eps, stream_));
+      }
+      norm_ready = false;
       LCU_CHECK(lcu_decode_qkv(t_xq_.data(), kc, vc, t_norm_.data(), nullptr, L.wq.data.data(), L.wk.data.data(),
                                L.wv.data.data(), L.wq.scales.data(), L.wk.scales.data(), L.wv.scales.data(), block, dim,
                                heads, 0, t_step_.data(), p.norm_eps, rope_table_, context_len_, stream_));
@@ -379,7 +384,16 @@ void llama_context_impl::enqueue_layers(int n) {
       matmul_multi(up_out, t_norm_.data(), up_w, 2, n);                                                      // 1180, 1181
       LCU_CHECK(lcu_silu_mul(t_silu_.data(), t_w1_.data(), t_w3_.data(), (size_t)n * ffn, stream_));         // 1183
     }
-    matmul(x, t_silu_.data(), L.w2, n, 1.0f);                                                                // 1185
+    if (n == 1 && l + 1 < model_->layers.size() && dim <= 8192) {
+      // 1185 and the next layer's 1129 in one launch
+      llama_layer const& next = model_->layers[l + 1];
+      LCU_CHECK(lcu_decode_proj_norm(x, t_norm_.data(), t_silu_.data(), L.w2.data.data(), L.w2.scales.data(), block,
+                                     ffn, dim, next.attn_norm.data(), p.norm_eps,
+                                     (char*)t_step_.data() + offsetof(step_state, seq), (int)(l & 1023), stream_));
+      norm_ready = true;
+    } else {
+      matmul(x, t_silu_.data(), L.w2, n, 1.0f);                                                              // 1185
+    }
   }
 }
 

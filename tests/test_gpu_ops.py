@@ -718,6 +718,80 @@ def test_decode_attention_wo_norm_equals_its_separate_operators(gpu, heads, ctx)
     G.release()
 
 
+@pytest.mark.parametrize("K,N,u8", [(11008, 4096, False), (17920, 6656, True), (4096, 4096, True), (2816, 1024, False),
+                                    (512, 8, False), (1024, 8192, False)])
+def test_decode_proj_norm_equals_its_separate_operators(gpu, K, N, u8):
+    """lcu_decode_proj_norm (x += lhs . W^T and the RMS norm of the new x in one launch; an extra workgroup waits
+    inside the launch for the rows) against lcu_gemm_* (beta 1) + lcu_rmsnorm and the kernel-order oracle, bit for
+    bit, eager and replayed from a graph with the step counter changed between replays."""
+    import ctypes as C
+    G = gpu
+    L = G.L()
+    eps = 1e-6
+    lhs = [normal((1, K), 0, 1400 + i, 1.0) for i in range(3)]
+    x0 = normal((1, N), 0, 1410, 1.0)
+    w, nw = normal((N, K), 0, 1411, 0.02), normal((N,), 1, 1412, 0.3)
+    block = 128 if u8 else 0
+    if u8:
+        codes, scales = O.quantize_absmax_u8(w, block)
+        wd, sd = G.dev_keep(codes), G.dev_keep(scales)
+    else:
+        wd, sd = G.dev_keep(w), None
+    nwd = G.dev_keep(nw)
+    lhs_d = G.empty((1, K))
+    x_f, n_f, x_s, n_s = G.empty((1, N)), G.empty((1, N)), G.empty((1, N)), G.empty((1, N))
+    stream = C.c_void_p()
+    G.B.check(L.lcu_stream_create(C.byref(stream)))
+    state = G.B.DeviceBuffer(8)
+    def prepare(seq, which):
+        a = np.array([0, seq], dtype=np.uint32)
+        G.B.check(L.lcu_h2d(state.ptr, a.ctypes.data_as(C.c_void_p), 8, stream))
+        G.B.check(L.lcu_h2d(lhs_d.ptr, lhs[which].ctypes.data_as(C.c_void_p), lhs[which].nbytes, stream))
+        for dst in (x_f, x_s):
+            G.B.check(L.lcu_h2d(dst.ptr, x0.ctypes.data_as(C.c_void_p), x0.nbytes, stream))
+        G.B.check(L.lcu_sync(stream))
+    def fused():
+        G.B.check(L.lcu_decode_proj_norm(x_f.ptr, n_f.ptr, lhs_d.ptr, wd.ptr, sd.ptr if u8 else None, block, K, N, nwd.ptr,
+                                         eps, state.ptr + 4, 3, stream))
+    def check(which):
+        if u8:
+            G.B.check(L.lcu_gemm_f16u8_nt(x_s.ptr, lhs_d.ptr, wd.ptr, sd.ptr, 1, K, N, block, 1.0, stream))
+        else:
+            G.B.check(L.lcu_gemm_f16_nt(x_s.ptr, lhs_d.ptr, wd.ptr, 1, K, N, 1.0, stream))
+        G.B.check(L.lcu_rmsnorm(n_s.ptr, x_s.ptr, nwd.ptr, 1, N, eps, stream))
+        G.B.check(L.lcu_sync(stream))
+        got_x, got_n = G.host(x_f, (1, N)), G.host(n_f, (1, N))
+        assert G.ulp_mismatch(got_x, G.host(x_s, (1, N))) == 0.0, which
+        assert G.ulp_mismatch(got_n, G.host(n_s, (1, N))) == 0.0, which
+        if u8:
+            want_x = O.matmul_nt_u8(lhs[which], codes, scales, block, beta=1.0, out=x0, flavour=2)
+        else:
+            want_x = O.matmul_nt(lhs[which], w, flavour=2, beta=1.0, out=x0)
+        assert G.ulp_mismatch(got_x, want_x) == 0.0, which
+        assert G.ulp_mismatch(got_n, O.rms_norm(want_x, nw, eps)) == 0.0, which
+    prepare(1, 0)
+    fused()
+    check(0)
+    prepare(2, 0)
+    G.B.check(L.lcu_graph_begin_capture(stream))
+    fused()
+    graph = C.c_void_p()
+    G.B.check(L.lcu_graph_end_capture(stream, C.byref(graph)))
+    for step in range(4):
+        prepare(3 + step, step % 3)
+        G.B.check(L.lcu_graph_launch(graph, stream))
+        check(step % 3)
+    count = C.c_uint(123)
+    G.B.check(L.lcu_sync_timeouts(stream, C.byref(count)))
+    assert count.value == 0
+    assert L.lcu_decode_proj_norm(x_f.ptr, n_f.ptr, lhs_d.ptr, wd.ptr, sd.ptr if u8 else None, block, K, 8200, nwd.ptr, eps,
+                                  state.ptr + 4, 3, stream) == -2
+    G.B.check(L.lcu_graph_destroy(graph))
+    G.B.check(L.lcu_stream_destroy(stream))
+    state.free()
+    G.release()
+
+
 @pytest.mark.parametrize("B,dim,heads,ffn,u8", [(8, 4096, 32, 11008, False), (8, 4096, 32, 11008, True), (33, 1024, 8, 2816, False),
                                                 (3, 320, 2, 704, False), (1, 512, 4, 1408, True)])
 def test_batch_fused_steps_equal_their_separate_operators(gpu, B, dim, heads, ffn, u8):

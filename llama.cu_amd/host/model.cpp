@@ -370,7 +370,12 @@ void llama_context_impl::enqueue_layers(int n) {
       LCU_CHECK(lcu_rope(k_new, k_new, n, dim, heads, sp, rope_table_, context_len_, stream_));  // 1152, new rows only
       LCU_CHECK(lcu_attention(t_out_.data(), t_xq_.data(), kc, vc, n, T, sp, dim, heads, stream_));          // 1161-1171
     }
-    if (!fused_wo) {
+    if (n == 1 && !fused_wo && dim <= 8192) {
+      // 1174 and 1176 in one launch (salts: even for this one, odd for the W2 launch below)
+      LCU_CHECK(lcu_decode_proj_norm(x, t_norm_.data(), t_out_.data(), L.wo.data.data(), L.wo.scales.data(), block, dim,
+                                     dim, L.ffn_norm.data(), p.norm_eps,
+                                     (char*)t_step_.data() + offsetof(step_state, seq), (int)((2 * l) & 1023), stream_));
+    } else if (!fused_wo) {
       matmul(x, t_out_.data(), L.wo, n, 1.0f);                                                               // 1174
       LCU_CHECK(lcu_rmsnorm(t_norm_.data(), x, L.ffn_norm.data(), n, dim, p.norm_eps, stream_));             // 1176
     }
@@ -389,7 +394,7 @@ void llama_context_impl::enqueue_layers(int n) {
       llama_layer const& next = model_->layers[l + 1];
       LCU_CHECK(lcu_decode_proj_norm(x, t_norm_.data(), t_silu_.data(), L.w2.data.data(), L.w2.scales.data(), block,
                                      ffn, dim, next.attn_norm.data(), p.norm_eps,
-                                     (char*)t_step_.data() + offsetof(step_state, seq), (int)(l & 1023), stream_));
+                                     (char*)t_step_.data() + offsetof(step_state, seq), (int)((2 * l + 1) & 1023), stream_));
       norm_ready = true;
     } else {
       matmul(x, t_silu_.data(), L.w2, n, 1.0f);                                                              // 1185

@@ -243,8 +243,19 @@ llama_context_impl::llama_context_impl(llama_model* model, int context_len, floa
   clear_tokens();
 }
 
+void llama_context_impl::check_hand_overs() {
+  unsigned timeouts = 0;
+  LCU_CHECK(lcu_sync_timeouts(stream_, &timeouts));
+  if (timeouts != 0) {
+    fprintf(stderr, "%u hand-overs between workgroups of a decode launch did not arrive: the results of this context "
+                    "are not to be trusted (is other work holding compute units of this device?)\n", timeouts);
+    raise(SIGSEGV);
+  }
+}
+
 llama_context_impl::~llama_context_impl() {
   lcu_sync(stream_);
+  check_hand_overs();
   lcu_graph_destroy(decode_graph_);
   lcu_free(rope_table_);
   lcu_stream_destroy(stream_);
@@ -536,6 +547,12 @@ short llama_context_impl::next_token(std::vector<short> const& new_tokens) {
   }
   int token = 0;
   LCU_CHECK(lcu_d2h(&token, t_argmax_.data(), sizeof(int), stream_));  // 1198-1200, blocks
+  // The one-token launches hand results over between their workgroups with bounded waits; a wait that
+  // ran out leaves a wrong result behind, which is a device error like any other: fatal.  Looked at
+  // every 32 steps (4 bytes back) and when the context goes away.
+  if (n == 1 && (decode_calls_ & 31) == 0) {
+    check_hand_overs();
+  }
   start_pos_ += n;
   last_n_ = n;
   return (short)token;

@@ -78,6 +78,7 @@ struct llama_context_impl final : public llama_context {
   void enqueue_layers(int n);
   void enqueue_head(int n);
   void drop_graph();
+  void check_hand_overs();
   std::vector<kv_cache_layer> kv_;
   gpu_buffer t_embed_, t_norm_, t_xq_, t_out_, t_w1_, t_w3_, t_silu_;
   gpu_buffer t_tokens_, t_logits_, t_probs_, t_argmax_;

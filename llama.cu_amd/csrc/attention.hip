@@ -294,13 +294,6 @@ __global__ __launch_bounds__(256) void dec_softmax_pv_kernel(half_t* __restrict_
 constexpr int SPREAD = 8;
 constexpr int SPREAD_SPIN_LIMIT = 1 << 16;
 
-// the wait for it is the caller's (s_waitcnt vmcnt(0) after the last of a group)
-__device__ __forceinline__ uint64_t request_u64_device_scope(const uint64_t* p) {
-  uint64_t v;
-  asm volatile("global_load_dwordx2 %0, %1, off sc0 sc1" : "=v"(v) : "v"(p) : "memory");
-  return v;
-}
-
 template <int NJ>
 __global__ __launch_bounds__(256) void decode_attention_spread_kernel(
     half_t* __restrict__ out, const half_t* __restrict__ q, const half_t* __restrict__ k, const half_t* __restrict__ v,
@@ -363,17 +356,20 @@ __global__ __launch_bounds__(256) void decode_attention_spread_kernel(
     uint64_t raw[NJ];
     int spins = 0;
     while (true) {
+      // four words per statement; an element past T reads word 0 of the row instead and is ignored
 #pragma unroll
-      for (int j = 0; j < NJ; ++j) {
-        raw[j] = tid + 256 * j < T ? request_u64_device_scope(srow + tid + 256 * j) : ((uint64_t)epoch << 32) | 0xfc00u;
+      for (int j = 0; j < NJ; j += 4) {
+        uint64_t four[4];
+        load_words_device_scope(four, srow + (tid + 256 * j < T ? tid + 256 * j : 0),
+                                srow + (tid + 256 * (j + 1) < T ? tid + 256 * (j + 1) : 0),
+                                srow + (tid + 256 * (j + 2) < T ? tid + 256 * (j + 2) : 0),
+                                srow + (tid + 256 * (j + 3) < T ? tid + 256 * (j + 3) : 0));
+#pragma unroll
+        for (int e = 0; e < 4; ++e) raw[j + e] = tid + 256 * (j + e) < T ? four[e] : ((uint64_t)epoch << 32) | 0xfc00u;
       }
-      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
       bool stale = false;
 #pragma unroll
-      for (int j = 0; j < NJ; ++j) {
-        asm volatile("" : "+v"(raw[j]));  // read only after the wait
-        stale |= (uint32_t)(raw[j] >> 32) != epoch;
-      }
+      for (int j = 0; j < NJ; ++j) stale |= (uint32_t)(raw[j] >> 32) != epoch;
       if (__builtin_amdgcn_ballot_w64(stale) == 0) break;
       if (++spins > SPREAD_SPIN_LIMIT) {
         if ((tid & 63) == 0) atomicAdd(timeouts, 1u);
@@ -453,25 +449,17 @@ constexpr int FUSED_PAD_LDS = 72 << 10;  // dynamic LDS nobody touches: a second
 
 static_assert(EXCH_ATT == MAX_HEADS * MAX_T_DECODE, "the scores' area");
 
-__device__ __forceinline__ uint4_t request_u128_device_scope(const void* p) {
-  uint4_t v;
-  asm volatile("global_load_dwordx4 %0, %1, off sc0 sc1" : "=v"(v) : "v"(p) : "memory");
-  return v;
-}
-
 // All threads of the workgroup: waits until the dim / 2 {half2, epoch} words at `words` carry this
 // launch's epoch and copies their halves to xs[0 .. dim).  Every thread asks for two words at a time.
 __device__ __forceinline__ void gather_row(half_t* xs, const uint64_t* words, int dim, uint32_t epoch,
                                            uint32_t* timeouts) {
   const int tid = threadIdx.x;
   for (int w0 = tid * 2; w0 < dim / 2; w0 += FUSED_THREADS * 2) {
-    uint4_t raw;
+    uint4_t raw[1];
     int spins = 0;
     while (true) {
-      raw = request_u128_device_scope(words + w0);
-      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-      asm volatile("" : "+v"(raw));  // read only after the wait
-      const bool stale = raw[1] != epoch || raw[3] != epoch;
+      load_word_pairs_device_scope(raw, words + w0);
+      const bool stale = raw[0][1] != epoch || raw[0][3] != epoch;
       if (__builtin_amdgcn_ballot_w64(stale) == 0) break;
       if (++spins > SPREAD_SPIN_LIMIT) {
         if ((tid & 63) == 0) atomicAdd(timeouts, 1u);
@@ -480,8 +468,8 @@ __device__ __forceinline__ void gather_row(half_t* xs, const uint64_t* words, in
       __builtin_amdgcn_s_sleep(1);
     }
     uint32_t* dst = reinterpret_cast<uint32_t*>(xs + 2 * w0);
-    dst[0] = raw[0];
-    dst[1] = raw[2];
+    dst[0] = raw[0][0];
+    dst[1] = raw[0][2];
   }
 }
 
@@ -589,17 +577,20 @@ __global__ __launch_bounds__(FUSED_THREADS) void decode_attention_wo_norm_kernel
     uint64_t raw[NJ];
     int spins = 0;
     while (true) {
+      // four words per statement; an element past T reads word 0 of the row instead and is ignored
 #pragma unroll
-      for (int j = 0; j < NJ; ++j) {
-        raw[j] = tid + 256 * j < T ? request_u64_device_scope(srow + tid + 256 * j) : ((uint64_t)epoch << 32) | 0xfc00u;
+      for (int j = 0; j < NJ; j += 4) {
+        uint64_t four[4];
+        load_words_device_scope(four, srow + (tid + 256 * j < T ? tid + 256 * j : 0),
+                                srow + (tid + 256 * (j + 1) < T ? tid + 256 * (j + 1) : 0),
+                                srow + (tid + 256 * (j + 2) < T ? tid + 256 * (j + 2) : 0),
+                                srow + (tid + 256 * (j + 3) < T ? tid + 256 * (j + 3) : 0));
+#pragma unroll
+        for (int e = 0; e < 4; ++e) raw[j + e] = tid + 256 * (j + e) < T ? four[e] : ((uint64_t)epoch << 32) | 0xfc00u;
       }
-      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
       bool stale = false;
 #pragma unroll
-      for (int j = 0; j < NJ; ++j) {
-        asm volatile("" : "+v"(raw[j]));
-        stale |= (uint32_t)(raw[j] >> 32) != epoch;
-      }
+      for (int j = 0; j < NJ; ++j) stale |= (uint32_t)(raw[j] >> 32) != epoch;
       if (__builtin_amdgcn_ballot_w64(stale) == 0) break;
       if (++spins > SPREAD_SPIN_LIMIT) {
         if (lane == 0) atomicAdd(timeouts, 1u);

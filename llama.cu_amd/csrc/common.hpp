@@ -233,6 +233,41 @@ __device__ __forceinline__ float block256_max(float v, float* red) {
   return fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
 }
 
+// ---- hand-over words read at device scope ----
+// Loads that bypass the caches another XCD's store does not reach (sc0 sc1), several at a time, and
+// the wait for them, in ONE asm statement: when the statement ends the data is in the registers, so
+// whatever the compiler does with those registers afterwards (copy, spill, reuse) is safe.  With the
+// wait in a statement of its own, the compiler -- which does not know that the registers are still
+// being written -- may reuse or spill them in between, and the data then lands on something else.
+// Early-clobber outputs: a register written by the first load must not hold a later load's address.
+// (The compiler's own device-scope atomic loads are safe too, but it issues them one by one with a
+// wait each: 1.7 us more per decoded layer.)
+__device__ __forceinline__ void load_words_device_scope(uint64_t (&o)[1], const uint64_t* p0) {
+  asm volatile("global_load_dwordx2 %0, %1, off sc0 sc1\n\ts_waitcnt vmcnt(0)" : "=&v"(o[0]) : "v"(p0) : "memory");
+}
+__device__ __forceinline__ void load_words_device_scope(uint64_t (&o)[4], const uint64_t* p0, const uint64_t* p1,
+                                                        const uint64_t* p2, const uint64_t* p3) {
+  asm volatile(
+      "global_load_dwordx2 %0, %4, off sc0 sc1\n\tglobal_load_dwordx2 %1, %5, off sc0 sc1\n\t"
+      "global_load_dwordx2 %2, %6, off sc0 sc1\n\tglobal_load_dwordx2 %3, %7, off sc0 sc1\n\ts_waitcnt vmcnt(0)"
+      : "=&v"(o[0]), "=&v"(o[1]), "=&v"(o[2]), "=&v"(o[3])
+      : "v"(p0), "v"(p1), "v"(p2), "v"(p3)
+      : "memory");
+}
+// two neighbouring words (16 bytes, 16-byte aligned) per request
+__device__ __forceinline__ void load_word_pairs_device_scope(uint4_t (&o)[1], const uint64_t* p0) {
+  asm volatile("global_load_dwordx4 %0, %1, off sc0 sc1\n\ts_waitcnt vmcnt(0)" : "=&v"(o[0]) : "v"(p0) : "memory");
+}
+__device__ __forceinline__ void load_word_pairs_device_scope(uint4_t (&o)[4], const uint64_t* p0, const uint64_t* p1,
+                                                             const uint64_t* p2, const uint64_t* p3) {
+  asm volatile(
+      "global_load_dwordx4 %0, %4, off sc0 sc1\n\tglobal_load_dwordx4 %1, %5, off sc0 sc1\n\t"
+      "global_load_dwordx4 %2, %6, off sc0 sc1\n\tglobal_load_dwordx4 %3, %7, off sc0 sc1\n\ts_waitcnt vmcnt(0)"
+      : "=&v"(o[0]), "=&v"(o[1]), "=&v"(o[2]), "=&v"(o[3])
+      : "v"(p0), "v"(p1), "v"(p2), "v"(p3)
+      : "memory");
+}
+
 // fp16((code - 127.5) * scale): the product is exact in fp32 (9 x 11 significant bits), so this
 // is one rounding, as dequantize_absmax_one (llama_cu.cu:287-289).
 __device__ __forceinline__ half_t dequant_one(uint32_t code, float scale) {

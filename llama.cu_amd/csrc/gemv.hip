@@ -564,24 +564,24 @@ __global__ __launch_bounds__(GEMV_THREADS) void decode_proj_norm_kernel(
     return;
   }
   const int tid = threadIdx.x;
+  // two neighbouring words per request, four requests per statement; a piece past the row reads the
+  // row's first words instead and is ignored
   uint4_t raw[FOLLOW_PIECES];
   int spins = 0;
   while (true) {
-#pragma unroll
-    for (int j = 0; j < FOLLOW_PIECES; ++j) {
-      const int w0 = (tid + GEMV_THREADS * j) * 2;
-      if (w0 < N / 2) {
-        asm volatile("global_load_dwordx4 %0, %1, off sc0 sc1" : "=v"(raw[j]) : "v"(words + w0) : "memory");
-      }
-    }
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     bool stale = false;
 #pragma unroll
-    for (int j = 0; j < FOLLOW_PIECES; ++j) {
-      const int w0 = (tid + GEMV_THREADS * j) * 2;
-      if (w0 < N / 2) {
-        asm volatile("" : "+v"(raw[j]));  // read only after the wait
-        stale |= raw[j][1] != epoch || raw[j][3] != epoch;
+    for (int j = 0; j < FOLLOW_PIECES; j += 4) {
+      if (GEMV_THREADS * j * 2 >= N / 2) continue;  // the whole group lies past the row (the same for every thread)
+      uint4_t four[4];
+      const int w0 = (tid + GEMV_THREADS * j) * 2, w1 = w0 + GEMV_THREADS * 2, w2 = w1 + GEMV_THREADS * 2,
+                w3 = w2 + GEMV_THREADS * 2;
+      load_word_pairs_device_scope(four, words + (w0 < N / 2 ? w0 : 0), words + (w1 < N / 2 ? w1 : 0),
+                                   words + (w2 < N / 2 ? w2 : 0), words + (w3 < N / 2 ? w3 : 0));
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        raw[j + e] = four[e];
+        if ((tid + GEMV_THREADS * (j + e)) * 2 < N / 2) stale |= four[e][1] != epoch || four[e][3] != epoch;
       }
     }
     if (__builtin_amdgcn_ballot_w64(stale) == 0) break;

@@ -722,7 +722,16 @@ __global__ __launch_bounds__(FUSED_THREADS) void decode_attention_wo_norm_kernel
   __syncthreads();  // (8)
   float sq = 0.0f;
   if (att) {
-    for (int i = tid; i < dim; i += 256) {
+    // eight LDS reads in flight at a time; the additions stay in ascending order
+    int i = tid;
+    for (; i + 7 * 256 < dim; i += 8 * 256) {
+      float e[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) e[u] = (float)xs[i + u * 256];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) sq = fmaf(e[u], e[u], sq);
+    }
+    for (; i < dim; i += 256) {
       const float e = (float)xs[i];
       sq = fmaf(e, e, sq);
     }

@@ -589,7 +589,7 @@ __global__ __launch_bounds__(GEMV_THREADS) void decode_proj_norm_kernel(
       if ((tid & 63) == 0) atomicAdd(timeouts, 1u);
       break;
     }
-    __builtin_amdgcn_s_sleep(8);
+    __builtin_amdgcn_s_sleep(2);
   }
 #pragma unroll
   for (int j = 0; j < FOLLOW_PIECES; ++j) {
@@ -603,9 +603,20 @@ __global__ __launch_bounds__(GEMV_THREADS) void decode_proj_norm_kernel(
   __syncthreads();
   // rms_norm, llama_cu.cu:66-107, as rmsnorm_kernel: thread t owns elements t, t + 256, ...
   float s = 0.0f;
-  for (int i = tid; i < N; i += GEMV_THREADS) {
-    const float e = (float)xs[i];
-    s = fmaf(e, e, s);
+  {
+    // eight LDS reads in flight at a time; the additions stay in ascending order
+    int i = tid;
+    for (; i + 7 * GEMV_THREADS < N; i += 8 * GEMV_THREADS) {
+      float e[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) e[u] = (float)xs[i + u * GEMV_THREADS];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) s = fmaf(e[u], e[u], s);
+    }
+    for (; i < N; i += GEMV_THREADS) {
+      const float e = (float)xs[i];
+      s = fmaf(e, e, s);
+    }
   }
   const float total = block256_sum_ref_order_dpp(s, red);
   const float rms_inv = 1.0f / sqrtf(total / (float)N + eps);

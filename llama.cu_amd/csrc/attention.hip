@@ -507,6 +507,12 @@ __global__ __launch_bounds__(FUSED_THREADS) void decode_attention_wo_norm_kernel
   if (pos_dev) T = min(max(*pos_dev + 1, 1), T_cap);
   if (seq_dev) epoch = (epoch | (*seq_dev << 10)) & 0x7fffffffu;
   uint64_t* srow = exch + (size_t)h * T_cap;
+  // what the 16 finishing threads need from memory at the very end, requested now
+  half_t x_old = (half_t)0.0f, nw_mine = (half_t)0.0f;
+  if (tid < 16) {
+    x_old = x_io[row0 + tid];
+    nw_mine = norm_w[row0 + tid];
+  }
 
   // ---- this workgroup's rows of Wo live in the registers of wavefronts 4-15: row team - 1 + 3 i of
   // the 16 goes to the four wavefronts of `team` (1..3).  The requests go out in four batches, one
@@ -711,7 +717,7 @@ __global__ __launch_bounds__(FUSED_THREADS) void decode_attention_wo_norm_kernel
     float acc = 0.0f;
 #pragma unroll
     for (int w = 0; w < 4; ++w) acc += part[tid][w];
-    const half_t xn = round_f16(fmaf(1.0f, (float)x_io[row0 + tid], acc));  // llama_cu.cu:279 with beta = 1
+    const half_t xn = round_f16(fmaf(1.0f, (float)x_old, acc));  // llama_cu.cu:279 with beta = 1
     x_io[row0 + tid] = xn;
     publish16(exch + EXCH_X, row0, xn, epoch);
   }
@@ -753,7 +759,7 @@ __global__ __launch_bounds__(FUSED_THREADS) void decode_attention_wo_norm_kernel
     const float total = ((lo[0] + hi[0]) + (lo[2] + hi[2])) + ((lo[1] + hi[1]) + (lo[3] + hi[3]));
     const float rms_inv = 1.0f / sqrtf(total / (float)dim + eps);
     const half_t inner = round_f16((float)xs[row0 + tid] * rms_inv);
-    norm_out[row0 + tid] = round_f16((float)norm_w[row0 + tid] * (float)inner);
+    norm_out[row0 + tid] = round_f16((float)nw_mine * (float)inner);
   }
 }
 

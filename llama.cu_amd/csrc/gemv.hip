@@ -564,6 +564,13 @@ __global__ __launch_bounds__(GEMV_THREADS) void decode_proj_norm_kernel(
     return;
   }
   const int tid = threadIdx.x;
+  // the norm weights of this thread's pieces, requested before the wait (N <= 8192: four pieces)
+  half8_t nwp[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int i = (tid + GEMV_THREADS * j) * 8;
+    nwp[j] = i < N ? *reinterpret_cast<const half8_t*>(norm_w + i) : (half8_t)(0.0f);
+  }
   // two neighbouring words per request, four requests per statement; a piece past the row reads the
   // row's first words instead and is ignored
   uint4_t raw[FOLLOW_PIECES];
@@ -620,9 +627,12 @@ __global__ __launch_bounds__(GEMV_THREADS) void decode_proj_norm_kernel(
   }
   const float total = block256_sum_ref_order_dpp(s, red);
   const float rms_inv = 1.0f / sqrtf(total / (float)N + eps);
-  for (int i = tid * 8; i < N; i += GEMV_THREADS * 8) {
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int i = (tid + GEMV_THREADS * j) * 8;
+    if (i >= N) continue;
     const half8_t xv = *reinterpret_cast<const half8_t*>(xs + i);
-    const half8_t wv = *reinterpret_cast<const half8_t*>(norm_w + i);
+    const half8_t wv = nwp[j];
     half8_t r;
 #pragma unroll
     for (int e = 0; e < 8; ++e) {

@@ -12,6 +12,8 @@
 #include <stdlib.h>
 #include <string.h>
 
+#include <mutex>
+
 #include "model_impl.hpp"
 
 namespace llama_cu {
@@ -517,6 +519,15 @@ short llama_context_impl::next_token(std::vector<short> const& new_tokens) {
     enqueue_layers(n);
     enqueue_head(n);
   };
+  // One decode step at a time per process: the launch that joins attention, Wo and norm puts one
+  // workgroup on every compute unit and these wait for one another, so two such launches running side
+  // by side (two contexts driven from two host threads) could each hold compute units the other needs
+  // until their bounded waits run out.  Held from the launch to the token's arrival.
+  static std::mutex decode_step_mutex;
+  std::unique_lock<std::mutex> one_step(decode_step_mutex, std::defer_lock);
+  if (n == 1) {
+    one_step.lock();
+  }
   if (n == 1) {
     // A decode step is ~260 launches of a few microseconds each: the first one runs eagerly (and
     // loads the kernels), the second is captured into a HIP graph, every later one replays it.

@@ -361,6 +361,38 @@ def test_context_api_behaviour(gpu):
     assert c.memory_usage() > 2 * 2 * 8 * 256 * 2
 
 
+def test_two_contexts_decoding_from_two_threads(gpu):
+    """Two contexts of one model driven from two host threads at once: the decode launch that joins attention,
+    Wo and norm holds every compute unit and its workgroups wait for one another, so the host layer lets one
+    decode step run at a time; both threads must get the tokens they get alone."""
+    import threading
+    G = gpu
+    cfg = dict(dim=4096, multiple_of=256, n_heads=32, n_layers=2, n_vocab=512, norm_eps=1e-6, q_type=0, qblock=128)
+    gm = G.P.Model(**cfg, seed=5)
+    prompts = [[3, 7, 11, 200, 5], [9, 8, 401, 2]]
+    steps = 40
+
+    def generate(i, out):
+        c = G.P.Context(gm, context_len=128, temperature=0.8)
+        toks = [c.next_token(prompts[i])]
+        for _ in range(steps):
+            toks.append(c.next_token([toks[-1]]))
+        out[i] = toks
+        c.close()
+
+    alone = [None, None]
+    for i in range(2):
+        generate(i, alone)
+    together = [None, None]
+    threads = [threading.Thread(target=generate, args=(i, together)) for i in range(2)]
+    for th in threads:
+        th.start()
+    for th in threads:
+        th.join()
+    assert together == alone
+    gm.close()
+
+
 def test_context_length_limits(gpu):
     """The attention kernels bound the context length: a longer one is refused when the context is
     created (the reference leaves it free, llama_cu.h:376), never in the middle of a generation."""

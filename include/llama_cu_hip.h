@@ -183,6 +183,8 @@ int lcu_attention_decode_spread(void* out_dev, const void* q_dev, const void* k_
  * 8 * n_heads workgroups wait for one another and must all be resident, one per compute unit: more
  * heads than a eighth of the compute units are refused (LCU_E_SHAPE), and on a device whose compute
  * units other work holds for good the waits run out (lcu_sync_timeouts) and the result is undefined.
+ * Two launches of this entry point must not run at the same time (two streams): each could hold compute
+ * units the other is waiting for; the host layer runs one decode step at a time for that reason.
  * x_io_dev: the residual row, updated in place. */
 int lcu_decode_attention_wo_norm(void* x_io_dev, void* norm_out_dev, const void* q_dev, const void* k_dev,
                                  const void* v_dev, const void* wo_dev, const void* norm_w_dev, float eps,

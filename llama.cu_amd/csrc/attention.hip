@@ -1172,21 +1172,13 @@ int lcu_decode_attention_wo_norm(void* x_io_dev, void* norm_out_dev, const void*
   if (!attr_set[dev & 15]) {
     LCU_HIP(hipFuncSetAttribute((const void*)decode_attention_wo_norm_kernel<1>,
                                 hipFuncAttributeMaxDynamicSharedMemorySize, FUSED_PAD_LDS));
-    LCU_HIP(hipFuncSetAttribute((const void*)decode_attention_wo_norm_kernel<2>,
-                                hipFuncAttributeMaxDynamicSharedMemorySize, FUSED_PAD_LDS));
     attr_set[dev & 15] = true;
   }
-  if (dim <= 4096) {
-    decode_attention_wo_norm_kernel<1><<<grid, FUSED_THREADS, FUSED_PAD_LDS, s>>>(
-        (half_t*)x_io_dev, (half_t*)norm_out_dev, (const half_t*)q_dev, (const half_t*)k_dev, (const half_t*)v_dev,
-        (const half_t*)wo_dev, (const half_t*)norm_w_dev, eps, max_T, dim, n_heads, (const int*)pos_dev, exch,
-        (const uint32_t*)seq_dev, (uint32_t)salt, ws.sync + SYNC_TIMEOUTS);
-  } else {
-    decode_attention_wo_norm_kernel<2><<<grid, FUSED_THREADS, FUSED_PAD_LDS, s>>>(
-        (half_t*)x_io_dev, (half_t*)norm_out_dev, (const half_t*)q_dev, (const half_t*)k_dev, (const half_t*)v_dev,
-        (const half_t*)wo_dev, (const half_t*)norm_w_dev, eps, max_T, dim, n_heads, (const int*)pos_dev, exch,
-        (const uint32_t*)seq_dev, (uint32_t)salt, ws.sync + SYNC_TIMEOUTS);
-  }
+  LCU_REQUIRE(dim <= 4096, "lcu_decode_attention_wo_norm: dim %d beyond 4096", dim);  // 32 heads of 128
+  decode_attention_wo_norm_kernel<1><<<grid, FUSED_THREADS, FUSED_PAD_LDS, s>>>(
+      (half_t*)x_io_dev, (half_t*)norm_out_dev, (const half_t*)q_dev, (const half_t*)k_dev, (const half_t*)v_dev,
+      (const half_t*)wo_dev, (const half_t*)norm_w_dev, eps, max_T, dim, n_heads, (const int*)pos_dev, exch,
+      (const uint32_t*)seq_dev, (uint32_t)salt, ws.sync + SYNC_TIMEOUTS);
   LCU_LAUNCH_CHECK();
   return LCU_OK;
 }

@@ -61,6 +61,12 @@ int lcu_stream_create(void** out_stream);
 int lcu_stream_destroy(void* stream);
 /* bounded in-launch waits that ran out on this stream's workspace so far (0 in any healthy run) */
 int lcu_sync_timeouts(void* stream, unsigned* out_count);
+
+/* Clears the stream's hand-over words (stream-ordered, not under capture).  A hand-over word is taken for new
+ * when it carries the launch's epoch, 21 bits of *seq_dev and the salt: a caller whose step counter has run
+ * through 2^21 values clears the words before the epochs repeat, and never uses a counter whose low 21 bits
+ * are zero with salt 0 (the epoch of a cleared word).  No counterpart in the reference. */
+int lcu_sync_reset(void* stream);
 int lcu_sync(void* stream);                                                     /* NULL = whole device */
 /* HIP graph capture of the launches made on `stream` between begin and end; every lcu_* kernel
  * entry point may be captured (none of them records a memset node or allocates).  No counterpart

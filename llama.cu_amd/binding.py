@@ -74,6 +74,7 @@ SIGNATURES = {
     "lcu_attention_decode": (i32, [vp, vp, vp, vp, vp, i32, i32, i32, vp]),
     "lcu_attention_decode_spread": (i32, [vp, vp, vp, vp, vp, vp, i32, i32, i32, i32, vp]),
     "lcu_sync_timeouts": (i32, [vp, vp]),
+    "lcu_sync_reset": (i32, [vp]),
     "lcu_decode_proj_norm": (i32, [vp, vp, vp, vp, vp, i32, i32, i32, vp, f32, vp, i32, vp]),
     "lcu_decode_attention_wo_norm": (i32, [vp, vp, vp, vp, vp, vp, vp, C.c_float, vp, vp, i32, i32, i32, i32, vp]),
     "lcu_graph_begin_capture": (i32, [vp]),

@@ -220,6 +220,17 @@ int lcu_sync_timeouts(void* stream, unsigned* out_count) {
   return LCU_OK;
 }
 
+int lcu_sync_reset(void* stream) {
+  const workspace_t ws = workspace_for(as_stream(stream));
+  if (ws.sync == nullptr) return set_error(LCU_E_NOINIT, "lcu_sync_reset: lcu_init has not run on this device");
+  hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+  if (stream) LCU_HIP(hipStreamIsCapturing(as_stream(stream), &capturing));
+  LCU_REQUIRE(capturing == hipStreamCaptureStatusNone, "lcu_sync_reset: the stream is capturing");
+  LCU_HIP(hipMemsetAsync(ws.sync + SYNC_EXCHANGE, 0, (size_t)(SYNC_WORDS - SYNC_EXCHANGE) * sizeof(uint32_t),
+                         as_stream(stream)));
+  return LCU_OK;
+}
+
 int lcu_sync(void* stream) {
   if (stream) {
     LCU_HIP(hipStreamSynchronize(as_stream(stream)));

@@ -500,7 +500,12 @@ short llama_context_impl::next_token(std::vector<short> const& new_tokens) {
     ++samples_drawn_;
   }
   if (n == 1 || sampling_) {
-    ++host_step_.seq;
+    // The launches that hand results over inside themselves tell new words from old ones by the low 21 bits of
+    // this counter: when those come round, the words are cleared, and the value that cleared words carry is skipped.
+    if ((++host_step_.seq & 0x1fffffu) == 0) {
+      ++host_step_.seq;
+      LCU_CHECK(lcu_sync_reset(stream_));
+    }
     LCU_CHECK(lcu_h2d(t_step_.data(), &host_step_, sizeof(host_step_), stream_));
   }
   if (n == 1) {

@@ -637,6 +637,19 @@ def test_attention_decode_spread_in_a_replayed_graph(gpu, heads, ctx):
             G.B.check(L.lcu_attention_decode(old.ptr, qd[i].ptr, kd[i].ptr, vd[i].ptr, state.ptr, ctx, dim, heads, stream))
             G.B.check(L.lcu_sync(stream))
             assert G.ulp_mismatch(got, G.host(old, (1, dim))) == 0.0, (pos, i)
+    # a step counter that has come round to the same low 21 bits: the caller clears the hand-over words first
+    G.B.check(L.lcu_sync_reset(stream))
+    set_state(300, 2 + (1 << 21))
+    G.B.check(L.lcu_graph_launch(graph, stream))
+    G.B.check(L.lcu_sync(stream))
+    for i in range(2):
+        assert G.ulp_mismatch(G.host(out[i], (1, dim)), O.attention_decode_kernel_order(q[i], k[i][:301], v[i][:301], heads)) == 0.0
+    G.B.check(L.lcu_graph_begin_capture(stream))
+    assert L.lcu_sync_reset(stream) == -2  # a memset node is not what a captured step may hold
+    enqueue()
+    graph2 = C.c_void_p()
+    G.B.check(L.lcu_graph_end_capture(stream, C.byref(graph2)))
+    G.B.check(L.lcu_graph_destroy(graph2))
     count = C.c_uint(123)
     G.B.check(L.lcu_sync_timeouts(stream, C.byref(count)))
     assert count.value == 0

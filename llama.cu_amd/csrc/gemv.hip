@@ -768,8 +768,9 @@ int lcu_decode_proj_norm(void* x_io_dev, void* norm_out_dev, const void* lhs_dev
   if (block > 0) {
     int rc = check_quant_args("lcu_decode_proj_norm", scales_dev, K, block);
     if (rc) return rc;
-    // rows per workgroup as gemv_u8 picks them
-    if (N >= 6144) {
+    // four rows per workgroup (x fetched half as often) where the rows are long; short rows (Wo) finish sooner
+    // as twice as many workgroups of two
+    if (N >= 6144 && K >= 8192) {
       decode_proj_norm_kernel<true, 4, 1><<<(N + 3) / 4 + 1, GEMV_THREADS, lds, st>>>(
           (half_t*)x_io_dev, (half_t*)norm_out_dev, (const half_t*)lhs_dev, w_dev, (const half_t*)scales_dev,
           (const half_t*)norm_w_dev, K, N, block, eps, words, (const uint32_t*)seq_dev, (uint32_t)salt, timeouts);

@@ -207,7 +207,8 @@ def gemm_leg(P, stream):
     for name, K, N, u8 in [("f16_512x4096x4096", 4096, 4096, False), ("f16_512x4096x11008", 4096, 11008, False),
                            ("f16_512x11008x4096", 11008, 4096, False), ("u8_512x4096x4096", 4096, 4096, True),
                            ("u8_512x4096x11008", 4096, 11008, True), ("u8_512x11008x4096", 11008, 4096, True)]:
-        copies = 4
+        # enough copies that neither the L2s nor the 256 MB memory-side cache can serve the weights
+        copies = max(4, -(-640 * 2**20 // (N * K * (1 if u8 else 2))))
         ws = []
         for c in range(copies):
             if u8:
@@ -235,7 +236,7 @@ def gemm_leg(P, stream):
             launch(i)
         t = Timer(B, stream)
         t.start()
-        iters = 50
+        iters = max(50, 2 * copies)
         for i in range(iters):
             launch(i)
         us = t.stop_ms() * 1e3 / iters

@@ -416,6 +416,30 @@ __global__ __launch_bounds__(64 * WM * WN * KS, WM * WN * KS <= 4 ? 2 : 1) void 
   }
   const int m0 = tm * BM, n0 = tn * BN;
 
+  // beta != 0: the old values of the output tile, asked for now in 16-byte pieces (tile row c / (BN / 8), eight
+  // columns from 8 (c % (BN / 8))) and handed to the lanes that need them through LDS after the last stage.
+  // Read lane by lane in the accumulators' layout (2-byte requests, two rows of 64 bytes per instruction) they cost
+  // the 512 x 4096 x 4096 product 6 us.  Rows of N % 8 != 0 are not 16-byte aligned: those keep the 2-byte reads.
+  // Only where a thread holds at most two pieces (the 128 x 64 tile of 512 threads, which carries Wo): the
+  // registers that more pieces occupy through the K loop cost the 256 x 128 tile 5 % with beta = 0.
+  constexpr int OC = BM * BN / 8 / THREADS;  // pieces per thread
+  constexpr int OLD_LD = BN + 8;             // halves per tile row in LDS
+  constexpr bool OLD_PIECES = !SPLIT && OC <= 2;
+  static_assert(BM * BN / 8 % THREADS == 0 && BM * OLD_LD * 2 <= LDS_BYTES, "old tile staging");
+  const bool old_by_pieces = OLD_PIECES && beta != 0.0f && N % 8 == 0;
+  uint4_t old_piece[OC];
+  if constexpr (OLD_PIECES) {
+    if (old_by_pieces) {
+#pragma unroll
+      for (int j = 0; j < OC; ++j) {
+        const int c = tid + j * THREADS;
+        const int gm = m0 + c / (BN / 8), gn = n0 + (c % (BN / 8)) * 8;
+        old_piece[j] = (uint4_t)(0u);
+        if (gm < M && gn < N) old_piece[j] = *reinterpret_cast<const uint4_t*>(out + (size_t)gm * N + gn);
+      }
+    }
+  }
+
   // loader: instruction j of this wavefront fills LDS bytes [(wave + j*NW) * 1024, +1024) of the
   // operand's region; lane l lands on tile row c / CR, chunk position c % CR, c = that index * 64 + l
   uint32_t a_off[PA], b_off[PB];
@@ -701,6 +725,18 @@ __global__ __launch_bounds__(64 * WM * WN * KS, WM * WN * KS <= 4 ? 2 : 1) void 
     }
   }
 
+  half_t* old_lds = reinterpret_cast<half_t*>(gemm_lds);
+  if constexpr (OLD_PIECES) {
+    if (old_by_pieces) {
+      if constexpr (KS == 2) __syncthreads();  // the partial sums above have been read
+#pragma unroll
+      for (int j = 0; j < OC; ++j) {
+        const int c = tid + j * THREADS;
+        *reinterpret_cast<uint4_t*>(old_lds + (c / (BN / 8)) * OLD_LD + (c % (BN / 8)) * 8) = old_piece[j];
+      }
+      __syncthreads();
+    }
+  }
   // epilogue as in gemm_kernel (llama_cu.cu:208-215)
   if (group == 0) {
 #pragma unroll
@@ -710,7 +746,8 @@ __global__ __launch_bounds__(64 * WM * WN * KS, WM * WN * KS <= 4 ? 2 : 1) void 
         const int gn = n0 + wn + j * 32 + (lane & 31);
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
-          const int gm = m0 + wm + i * 32 + (v >> 2) * 8 + (lane >> 5) * 4 + (v & 3);
+          const int lm = wm + i * 32 + (v >> 2) * 8 + (lane >> 5) * 4 + (v & 3);
+          const int gm = m0 + lm;
           if (gm < M && gn < N) {
             if constexpr (SPLIT) {
               part[((size_t)split * M + gm) * N + gn] = acc[i][j][v];
@@ -718,7 +755,8 @@ __global__ __launch_bounds__(64 * WM * WN * KS, WM * WN * KS <= 4 ? 2 : 1) void 
               half_t* p = out + (size_t)gm * N + gn;
               float val = acc[i][j][v];
               if (beta != 0.0f) {
-                val = fmaf(beta, (float)*p, val);
+                const half_t before = old_by_pieces ? old_lds[lm * OLD_LD + wn + j * 32 + (lane & 31)] : *p;
+                val = fmaf(beta, (float)before, val);
               }
               *p = round_f16(val);
             }

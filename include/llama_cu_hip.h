@@ -121,6 +121,10 @@ int lcu_rmsnorm(void* out_dev, const void* in_dev, const void* weights_dev, int 
 int lcu_rope_table_create(void** out_table_dev, int positions, int head_dim, float theta);
 int lcu_rope(void* out_dev, const void* in_dev, int rows, int cols, int n_heads, int pos_offset,
              const void* table_dev, int table_positions, void* stream);
+/* lcu_rope in place on two tensors of one shape in one launch: the new rows of Q and of K of a prompt
+ * (launch sites 1146 and 1152; the reference rotates the whole K cache into a scratch copy on every call) */
+int lcu_rope_pair(void* a_dev, void* b_dev, int rows, int cols, int n_heads, int pos_offset, const void* table_dev,
+                  int table_positions, void* stream);
 /* softmax_rows, llama_cu.cu:433-499 (launch sites 1166, 1196); in place allowed */
 int lcu_softmax_rows(void* out_dev, const void* in_dev, int rows, int w, float temp, void* stream);
 /* e^x on n fp32 values with the exponential that every softmax and SiLU of this library takes

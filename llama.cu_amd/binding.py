@@ -52,6 +52,7 @@ SIGNATURES = {
     "lcu_rmsnorm": (i32, [vp, vp, vp, i32, i32, f32, vp]),
     "lcu_rope_table_create": (i32, [C.POINTER(vp), i32, i32, f32]),
     "lcu_rope": (i32, [vp, vp, i32, i32, i32, i32, vp, i32, vp]),
+    "lcu_rope_pair": (i32, [vp, vp, i32, i32, i32, i32, vp, i32, vp]),
     "lcu_softmax_rows": (i32, [vp, vp, i32, i32, f32, vp]),
     "lcu_silu_mul": (i32, [vp, vp, vp, sz, vp]),
     "lcu_exp_f32": (i32, [vp, vp, sz, vp]),

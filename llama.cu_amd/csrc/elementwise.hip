@@ -121,6 +121,25 @@ __global__ void rope_kernel(half_t* out, const half_t* in, int rows, int cols, i
   *reinterpret_cast<half2_t*>(out + o) = w;
 }
 
+// the same for two tensors of one shape in place (the new rows of Q and of K, llama_cu.cu:1146 and 1152):
+// blockIdx.z picks the tensor, so a prompt pays one launch for both
+__global__ void rope_pair_kernel(half_t* a, half_t* b, int rows, int cols, int head_dim, int pos_offset,
+                                 const float2* __restrict__ table) {
+  const int pair = blockIdx.x * blockDim.x + threadIdx.x;
+  const int r = blockIdx.y;
+  if (pair * 2 >= cols) return;
+  half_t* x = blockIdx.z ? b : a;
+  const int c = pair * 2;
+  const float2 cs = table[(size_t)(pos_offset + r) * (head_dim / 2) + (c % head_dim) / 2];
+  const size_t o = (size_t)r * cols + c;
+  const half2_t v = *reinterpret_cast<const half2_t*>(x + o);
+  const float real = (float)v.x, imag = (float)v.y;
+  half2_t w;
+  w.x = round_f16(fmaf(real, cs.x, -(imag * cs.y)));
+  w.y = round_f16(fmaf(real, cs.y, imag * cs.x));
+  *reinterpret_cast<half2_t*>(x + o) = w;
+}
+
 // ---------------------------------------------------------------------------------------------
 // softmax_rows, llama_cu.cu:433-499.  One 256-thread block per row, thread t owns elements
 // t, t+256, ...; the exponential sum is associated as in the reference.
@@ -728,6 +747,22 @@ int lcu_rope(void* out_dev, const void* in_dev, int rows, int cols, int n_heads,
   dim3 grid((cols / 2 + 255) / 256, rows);
   rope_kernel<<<grid, 256, 0, as_stream(stream)>>>((half_t*)out_dev, (const half_t*)in_dev, rows, cols,
                                                    cols / n_heads, pos_offset, (const float2*)table_dev);
+  LCU_LAUNCH_CHECK();
+  return LCU_OK;
+}
+
+int lcu_rope_pair(void* a_dev, void* b_dev, int rows, int cols, int n_heads, int pos_offset, const void* table_dev,
+                  int table_positions, void* stream) {
+  LCU_REQUIRE(a_dev && b_dev && table_dev, "lcu_rope_pair: null pointer");
+  LCU_REQUIRE(rows >= 0 && cols > 0 && n_heads > 0 && cols % n_heads == 0 && (cols / n_heads) % 2 == 0,
+              "lcu_rope_pair: bad shape rows %d cols %d heads %d", rows, cols, n_heads);
+  LCU_REQUIRE(pos_offset >= 0 && pos_offset + rows <= table_positions,
+              "lcu_rope_pair: positions %d..%d outside the table of %d", pos_offset, pos_offset + rows, table_positions);
+  LCU_REQUIRE(rows <= 65535, "lcu_rope_pair: %d rows, a grid holds 65535", rows);
+  if (rows == 0) return LCU_OK;
+  dim3 grid((cols / 2 + 255) / 256, rows, 2);
+  rope_pair_kernel<<<grid, 256, 0, as_stream(stream)>>>((half_t*)a_dev, (half_t*)b_dev, rows, cols, cols / n_heads,
+                                                        pos_offset, (const float2*)table_dev);
   LCU_LAUNCH_CHECK();
   return LCU_OK;
 }

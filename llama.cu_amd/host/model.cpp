@@ -379,8 +379,7 @@ void llama_context_impl::enqueue_layers(int n) {
       void* const qkv_out[3] = {t_xq_.data(), k_new, v_new};
       weight_tensor const* const qkv_w[3] = {&L.wq, &L.wk, &L.wv};
       matmul_multi(qkv_out, t_norm_.data(), qkv_w, 3, n);                                                    // 1144, 1150, 1156
-      LCU_CHECK(lcu_rope(t_xq_.data(), t_xq_.data(), n, dim, heads, sp, rope_table_, context_len_, stream_));  // 1146
-      LCU_CHECK(lcu_rope(k_new, k_new, n, dim, heads, sp, rope_table_, context_len_, stream_));  // 1152, new rows only
+      LCU_CHECK(lcu_rope_pair(t_xq_.data(), k_new, n, dim, heads, sp, rope_table_, context_len_, stream_));  // 1146, 1152 (new rows only)
       LCU_CHECK(lcu_attention(t_out_.data(), t_xq_.data(), kc, vc, n, T, sp, dim, heads, stream_));          // 1161-1171
     }
     if (n == 1 && !fused_wo && dim <= 8192) {

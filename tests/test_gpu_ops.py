@@ -403,6 +403,13 @@ def test_rope_bit_exact(gpu, rows, pos):
     G.B.check(G.L().lcu_rope(xd.ptr, xd.ptr, rows, dim, heads, pos, tab, 2048, None))
     assert G.ulp_mismatch(G.host(xd, (rows, dim)), got) == 0.0
     assert G.L().lcu_rope(xd.ptr, xd.ptr, rows, dim, heads, 2048 - rows + 1, tab, 2048, None) == -2  # past the table
+    # two tensors in one launch
+    y = normal((rows, dim), 0, 601, 1.0)
+    ad, bd = G.dev(x), G.dev(y)
+    G.B.check(G.L().lcu_rope_pair(ad.ptr, bd.ptr, rows, dim, heads, pos, tab, 2048, None))
+    assert G.ulp_mismatch(G.host(ad, (rows, dim)), got) == 0.0
+    assert G.ulp_mismatch(G.host(bd, (rows, dim)), O.rotary(y, heads, pos_offset=pos)) == 0.0
+    assert G.L().lcu_rope_pair(ad.ptr, bd.ptr, rows, dim, heads, 2048 - rows + 1, tab, 2048, None) == -2
     G.release()
     G.L().lcu_free(tab)
 

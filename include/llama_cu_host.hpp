@@ -155,26 +155,25 @@ struct LLAMA_CU_API llama_tokenizer {
   void tokenize(std::string_view text, std::vector<short>& output);
 
  private:
-  struct piece {
-    int prev;
-    int next;
-    std::string_view text;
-  };
-  struct candidate {
+  // Segments of the text being tokenized, as parallel arrays indexed by segment: bytes
+  // [begin_[i], begin_[i] + bytes_[i]) of text_, neighbours to either side (-1 at the ends), and a
+  // version that goes up whenever the segment grows or is swallowed (bytes_ 0), so that a queued
+  // merge can tell whether both of its sides are still what they were when it was queued.
+  struct merge {
+    float score;
     int left;
     int right;
-    float score;
-    size_t size;
+    uint32_t left_version;
+    uint32_t right_version;
   };
-  struct worse {
-    bool operator()(candidate const& l, candidate const& r) const {
-      return (l.score < r.score) || (l.score == r.score && l.left > r.left);
-    }
-  };
-  void consider(int left, int right);
+  short find_piece(size_t begin, size_t bytes, float* score);
+  void queue_merge(int left, int right);
   llama_vocabulary const& vocab_;
-  std::vector<piece> pieces_;
-  std::priority_queue<candidate, std::vector<candidate>, worse> queue_;
+  std::string_view text_;
+  std::vector<uint32_t> begin_, bytes_, version_;
+  std::vector<int> left_of_, right_of_;
+  std::vector<merge> heap_;
+  std::string key_;
 };
 
 struct llama_model_impl;

@@ -60,6 +60,12 @@ int lcu_context_read_hidden(lcu_context*, uint16_t* out, int rows);
 int lcu_context_read_kv(lcu_context*, int layer, uint16_t* k_out, uint16_t* v_out, int T);
 /* the hipStream_t (as void*) the context launches on, for event timing */
 void* lcu_context_stream(lcu_context*);
+/* How many one-token steps of this context were computed a second time because hand-overs between the
+ * workgroups of a decode launch did not arrive in time (other work held compute units of the device).
+ * Such a step's first token is never returned; from the first such step on the context uses launches
+ * that wait for nobody (what LLAMA_CU_NO_HANDOVER=1 selects from the start).  0 on a device the
+ * process has to itself.  No counterpart in the reference. */
+int lcu_context_hand_over_fallbacks(lcu_context*);
 /* llama_context::sample_with_seed / greedy: draw the next tokens from the probabilities (the
  * sampler the reference leaves commented out, llama_cu.cu:1202-1203) or take the maximum again */
 void lcu_context_set_sampling(lcu_context*, int enabled, uint64_t seed);

@@ -61,6 +61,9 @@ int lcu_stream_create(void** out_stream);
 int lcu_stream_destroy(void* stream);
 /* bounded in-launch waits that ran out on this stream's workspace so far (0 in any healthy run) */
 int lcu_sync_timeouts(void* stream, unsigned* out_count);
+/* Adds `count` to that counter (stream-ordered), as a wait that ran out would: lets a caller rehearse its
+ * handling of a failed hand-over without making any kernel wait.  No counterpart in the reference. */
+int lcu_sync_add_timeouts(void* stream, unsigned count);
 
 /* Clears the stream's hand-over words (stream-ordered, not under capture).  A hand-over word is taken for new
  * when it carries the launch's epoch, 21 bits of *seq_dev and the salt: a caller whose step counter has run
@@ -145,6 +148,13 @@ int lcu_argmax_f16(void* out_index_dev, const void* values_dev, int n, void* str
  * 1205-1209 on its rounded output, in one launch; probs_dev must not alias logits_dev */
 int lcu_softmax_argmax(void* probs_dev, void* out_index_dev, const void* logits_dev, int n, float temp,
                        void* stream);
+/* lcu_softmax_argmax whose output is two int32: the index, then the stream's count of bounded in-launch
+ * waits that ran out (what lcu_sync_timeouts reads) as it stands when this launch runs.  A step that ends
+ * with this launch brings its own health back in the copy that fetches the token: a count that has moved
+ * since the last step means hand-over words of this step were stale and its token must not be used
+ * (the fail-loud rule of llama_cu.h:48-56 applied to the in-launch hand-overs). */
+int lcu_softmax_argmax_status(void* probs_dev, void* out_index2_dev, const void* logits_dev, int n, float temp,
+                              void* stream);
 
 /* the sampler the reference leaves commented out at llama_cu.cu:1202-1203
  * (std::discrete_distribution over the probabilities): int32 index i drawn with probability

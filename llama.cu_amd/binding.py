@@ -75,6 +75,8 @@ SIGNATURES = {
     "lcu_attention_decode": (i32, [vp, vp, vp, vp, vp, i32, i32, i32, vp]),
     "lcu_attention_decode_spread": (i32, [vp, vp, vp, vp, vp, vp, i32, i32, i32, i32, vp]),
     "lcu_sync_timeouts": (i32, [vp, vp]),
+    "lcu_sync_add_timeouts": (i32, [vp, u32]),
+    "lcu_softmax_argmax_status": (i32, [vp, vp, vp, i32, f32, vp]),
     "lcu_sync_reset": (i32, [vp]),
     "lcu_decode_proj_norm": (i32, [vp, vp, vp, vp, vp, i32, i32, i32, vp, f32, vp, i32, vp]),
     "lcu_decode_attention_wo_norm": (i32, [vp, vp, vp, vp, vp, vp, vp, C.c_float, vp, vp, i32, i32, i32, i32, vp]),
@@ -107,6 +109,7 @@ SIGNATURES = {
     "lcu_context_read_hidden": (i32, [vp, vp, i32]),
     "lcu_context_read_kv": (i32, [vp, i32, vp, vp, i32]),
     "lcu_context_stream": (vp, [vp]),
+    "lcu_context_hand_over_fallbacks": (i32, [vp]),
     "lcu_context_set_sampling": (None, [vp, i32, u64]),
     "lcu_batch_create": (vp, [vp, i32, i32, f32]),
     "lcu_batch_destroy": (None, [vp]),
@@ -293,6 +296,9 @@ class Context:
     @property
     def stream(self):
         return lib().lcu_context_stream(self.h)
+
+    def hand_over_fallbacks(self):
+        return lib().lcu_context_hand_over_fallbacks(self.h)
 
     def logits(self):
         out = np.empty(self.model.n_vocab, dtype=np.float16)

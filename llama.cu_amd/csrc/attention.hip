@@ -1069,8 +1069,10 @@ int lcu_attention(void* out_dev, const void* q_dev, const void* k_dev, const voi
     LCU_REQUIRE((size_t)n_heads * T * sizeof(half_t) <= ws.bytes, "lcu_attention: workspace too small");
     hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
     if (s != nullptr) LCU_HIP(hipStreamIsCapturing(s, &capturing));
-    if (capturing == hipStreamCaptureStatusNone && ws.sync != nullptr) {
-      // the epoch of this launch is drawn on the host, so the launch must not be replayed
+    if (capturing == hipStreamCaptureStatusNone && ws.sync != nullptr && ws.owned) {
+      // Only on a stream that owns its workspace: the default stream and foreign streams share the
+      // device's, where two overlapping calls would overwrite each other's hand-over words.
+      // The epoch of this launch is drawn on the host, so the launch must not be replayed.
       return launch_decode_attention_spread((half_t*)out_dev, (const half_t*)q_dev, (const half_t*)k_dev,
                                             (const half_t*)v_dev, nullptr, T, dim, n_heads, ws, nullptr, 0, s);
     }

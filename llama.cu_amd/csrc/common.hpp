@@ -63,6 +63,8 @@ struct workspace_t {
   // heads x 4096 scores, then three rows of 4096), which no other operator may write: a reader trusts
   // a word by its epoch.
   uint32_t* sync = nullptr;
+  // true for the workspace of a stream made by lcu_stream_create: nobody else's launches use it
+  bool owned = false;
 };
 constexpr int SYNC_EXCHANGE = 2048;
 // offsets (in 8-byte words) of the hand-over areas: decode attention scores (64 heads x 4096), then

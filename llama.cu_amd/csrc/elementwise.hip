@@ -266,7 +266,8 @@ __global__ __launch_bounds__(1024) void sample_row_kernel(int* __restrict__ inde
 // 256-thread reference kernel (per-thread partials, then wavefronts, then 16 wavefront sums in
 // order), which moves a probability by at most the last fp32 bit of the sum.
 __global__ __launch_bounds__(1024) void softmax_argmax_kernel(half_t* __restrict__ probs, int* __restrict__ index,
-                                                              const half_t* __restrict__ logits, int n, float temp) {
+                                                              const half_t* __restrict__ logits, int n, float temp,
+                                                              const uint32_t* __restrict__ status_in) {
   __shared__ float sred[16];
   __shared__ int sidx[16];
   // one row per workgroup (several rows: one sequence of a batch each)
@@ -359,6 +360,7 @@ __global__ __launch_bounds__(1024) void softmax_argmax_kernel(half_t* __restrict
         }
       }
       *index = idx == 0x7fffffff ? 0 : idx;
+      if (status_in) index[1] = (int)*status_in;
     }
     return;
   }
@@ -436,6 +438,7 @@ __global__ __launch_bounds__(1024) void softmax_argmax_kernel(half_t* __restrict
       }
     }
     *index = idx == 0x7fffffff ? 0 : idx;
+    if (status_in) index[1] = (int)*status_in;
   }
 }
 
@@ -793,7 +796,22 @@ int lcu_softmax_argmax(void* probs_dev, void* out_index_dev, const void* logits_
   LCU_REQUIRE(n > 0 && temp > 0.0f, "lcu_softmax_argmax: bad arguments n %d temp %f", n, (double)temp);
   LCU_REQUIRE(probs_dev != logits_dev, "lcu_softmax_argmax: probabilities may not overwrite the logits");
   softmax_argmax_kernel<<<1, 1024, 0, as_stream(stream)>>>((half_t*)probs_dev, (int*)out_index_dev,
-                                                          (const half_t*)logits_dev, n, temp);
+                                                          (const half_t*)logits_dev, n, temp, nullptr);
+  LCU_LAUNCH_CHECK();
+  return LCU_OK;
+}
+
+int lcu_softmax_argmax_status(void* probs_dev, void* out_index2_dev, const void* logits_dev, int n, float temp,
+                              void* stream) {
+  LCU_REQUIRE(probs_dev && out_index2_dev && logits_dev, "lcu_softmax_argmax_status: null pointer");
+  LCU_REQUIRE(n > 0 && temp > 0.0f, "lcu_softmax_argmax_status: bad arguments n %d temp %f", n, (double)temp);
+  LCU_REQUIRE(probs_dev != logits_dev, "lcu_softmax_argmax_status: probabilities may not overwrite the logits");
+  const workspace_t ws = workspace_for(as_stream(stream));
+  if (ws.sync == nullptr) {
+    return set_error(LCU_E_NOINIT, "lcu_softmax_argmax_status: lcu_init has not run on this device");
+  }
+  softmax_argmax_kernel<<<1, 1024, 0, as_stream(stream)>>>((half_t*)probs_dev, (int*)out_index2_dev,
+                                                          (const half_t*)logits_dev, n, temp, ws.sync + SYNC_TIMEOUTS);
   LCU_LAUNCH_CHECK();
   return LCU_OK;
 }
@@ -806,7 +824,7 @@ int lcu_softmax_argmax_rows(void* probs_dev, void* out_index_dev, const void* lo
   LCU_REQUIRE(probs_dev != logits_dev, "lcu_softmax_argmax_rows: probabilities may not overwrite the logits");
   if (rows == 0) return LCU_OK;
   softmax_argmax_kernel<<<rows, 1024, 0, as_stream(stream)>>>((half_t*)probs_dev, (int*)out_index_dev,
-                                                             (const half_t*)logits_dev, n, temp);
+                                                             (const half_t*)logits_dev, n, temp, nullptr);
   LCU_LAUNCH_CHECK();
   return LCU_OK;
 }

@@ -426,7 +426,9 @@ __global__ __launch_bounds__(64 * WM * WN * KS, WM * WN * KS <= 4 ? 2 : 1) void 
   constexpr int OLD_LD = BN + 8;             // halves per tile row in LDS
   constexpr bool OLD_PIECES = !SPLIT && OC <= 2;
   static_assert(BM * BN / 8 % THREADS == 0 && BM * OLD_LD * 2 <= LDS_BYTES, "old tile staging");
-  const bool old_by_pieces = OLD_PIECES && beta != 0.0f && N % 8 == 0;
+  // 16-byte requests: rows of a multiple of 8 halves from a 16-byte aligned base (anything else keeps
+  // the 2-byte reads of the epilogue)
+  const bool old_by_pieces = OLD_PIECES && beta != 0.0f && N % 8 == 0 && (reinterpret_cast<uintptr_t>(out) & 15) == 0;
   uint4_t old_piece[OC];
   if constexpr (OLD_PIECES) {
     if (old_by_pieces) {

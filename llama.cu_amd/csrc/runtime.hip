@@ -40,7 +40,7 @@ workspace_t workspace_for(hipStream_t stream) {
   if (st == nullptr || !st->ready) {
     return workspace_t{};
   }
-  return workspace_t{st->workspace, st->workspace_bytes, st->workspace_sync};
+  return workspace_t{st->workspace, st->workspace_bytes, st->workspace_sync, false};
 }
 
 device_state* current_device_state() {
@@ -54,6 +54,10 @@ device_state* current_device_state() {
 }  // namespace lcu
 
 using namespace lcu;
+
+namespace {
+__global__ void add_u32_kernel(uint32_t* word, uint32_t count) { atomicAdd(word, count); }
+}  // namespace
 
 extern "C" {
 
@@ -178,6 +182,7 @@ int lcu_stream_create(void** out_stream) {
     e = hipDeviceSynchronize();  // the clearing is done before any stream can use the flags
   }
   ws.sync = reinterpret_cast<uint32_t*>((char*)ws.ptr + ws.bytes);
+  ws.owned = true;
   if (e != hipSuccess) {
     (void)hipFree(ws.ptr);
     (void)hipStreamDestroy(s);
@@ -217,6 +222,14 @@ int lcu_sync_timeouts(void* stream, unsigned* out_count) {
   if (ws.sync == nullptr) return set_error(LCU_E_NOINIT, "lcu_sync_timeouts: lcu_init has not run on this device");
   LCU_HIP(hipMemcpyAsync(out_count, ws.sync + SYNC_TIMEOUTS, sizeof(unsigned), hipMemcpyDeviceToHost, as_stream(stream)));
   LCU_HIP(hipStreamSynchronize(as_stream(stream)));
+  return LCU_OK;
+}
+
+int lcu_sync_add_timeouts(void* stream, unsigned count) {
+  const workspace_t ws = workspace_for(as_stream(stream));
+  if (ws.sync == nullptr) return set_error(LCU_E_NOINIT, "lcu_sync_add_timeouts: lcu_init has not run on this device");
+  add_u32_kernel<<<1, 1, 0, as_stream(stream)>>>(ws.sync + SYNC_TIMEOUTS, count);
+  LCU_LAUNCH_CHECK();
   return LCU_OK;
 }
 

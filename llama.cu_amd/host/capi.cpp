@@ -223,6 +223,8 @@ int lcu_context_read_kv(lcu_context* c, int layer, uint16_t* k_out, uint16_t* v_
 
 void* lcu_context_stream(lcu_context* c) { return c->impl()->stream(); }
 
+int lcu_context_hand_over_fallbacks(lcu_context* c) { return c->impl()->hand_over_fallbacks(); }
+
 lcu_batch* lcu_batch_create(lcu_model* m, int n_sequences, int context_len, float temperature) {
   if (!m || n_sequences <= 0 || context_len <= 0 || !(temperature > 0.0f)) {
     return nullptr;

@@ -242,22 +242,25 @@ llama_context_impl::llama_context_impl(llama_model* model, int context_len, floa
   compute_units_ = props.compute_units;
   const int head_dim = model_->params.dim / model_->params.n_heads;
   LCU_CHECK(lcu_rope_table_create(&rope_table_, context_len_, head_dim, 10000.0f));  // theta: llama_cu.cu:374
+  // The decode launches that hand results over between their own workgroups need those workgroups
+  // resident together, which only a device that this process has to itself guarantees.
+  // LLAMA_CU_NO_HANDOVER=1 (a GPU shared with other processes) keeps every context on launches that
+  // never wait for one another: same results, about a sixth slower.
+  const char* no_hand_over = getenv("LLAMA_CU_NO_HANDOVER");
+  hand_overs_ = !(no_hand_over != nullptr && atoi(no_hand_over) != 0);
+  LCU_CHECK(lcu_sync_timeouts(stream_, &timeouts_seen_));
   clear_tokens();
-}
-
-void llama_context_impl::check_hand_overs() {
-  unsigned timeouts = 0;
-  LCU_CHECK(lcu_sync_timeouts(stream_, &timeouts));
-  if (timeouts != 0) {
-    fprintf(stderr, "%u hand-overs between workgroups of a decode launch did not arrive: the results of this context "
-                    "are not to be trusted (is other work holding compute units of this device?)\n", timeouts);
-    raise(SIGSEGV);
-  }
 }
 
 llama_context_impl::~llama_context_impl() {
   lcu_sync(stream_);
-  check_hand_overs();
+  // Every one-token step has looked at the count of hand-overs that did not arrive before it returned
+  // its token (next_token), so there is nothing left to judge here; a context whose steps had to be
+  // recomputed says so once more when it goes.
+  if (hand_over_fallbacks_ > 0) {
+    fprintf(stderr, "llama_context: %d decode step(s) of this context were recomputed after hand-overs inside a "
+                    "launch did not arrive\n", hand_over_fallbacks_);
+  }
   lcu_graph_destroy(decode_graph_);
   lcu_free(rope_table_);
   lcu_stream_destroy(stream_);
@@ -288,7 +291,7 @@ void llama_context_impl::clear_tokens() {
     t_tokens_ = gpu_buffer(ctx * sizeof(short));
     t_logits_ = gpu_buffer((size_t)p.n_vocab * 2);
     t_probs_ = gpu_buffer((size_t)p.n_vocab * 2);
-    t_argmax_ = gpu_buffer(sizeof(int));
+    t_argmax_ = gpu_buffer(2 * sizeof(int));  // {token, count of hand-overs that did not arrive}
     t_step_ = gpu_buffer(sizeof(step_state));
   }
   LCU_CHECK(lcu_sync(stream_));
@@ -363,8 +366,12 @@ void llama_context_impl::enqueue_layers(int n) {
       const void* seq = (char*)t_step_.data() + offsetof(step_state, seq);
       // fp16 weights and rows of up to 1024 scores: attention, the Wo product with the residual sum
       // (1174) and the norm that follows (1176) in one launch
-      fused_wo = !L.wo.quantised && decode_bound_ <= 1024 && heads * 8 <= compute_units_;
-      if (fused_wo) {
+      fused_wo = hand_overs_ && !L.wo.quantised && decode_bound_ <= 1024 && heads * 8 <= compute_units_;
+      if (!hand_overs_) {
+        // launches whose workgroups never wait for one another (1161-1171)
+        LCU_CHECK(lcu_attention_decode(t_out_.data(), t_xq_.data(), kc, vc, t_step_.data(), decode_bound_, dim, heads,
+                                       stream_));
+      } else if (fused_wo) {
         LCU_CHECK(lcu_decode_attention_wo_norm(x, t_norm_.data(), t_xq_.data(), kc, vc, L.wo.data.data(),
                                                L.ffn_norm.data(), p.norm_eps, t_step_.data(), seq, (int)(l & 1023),
                                                decode_bound_, dim, heads, stream_));
@@ -382,7 +389,7 @@ void llama_context_impl::enqueue_layers(int n) {
       LCU_CHECK(lcu_rope_pair(t_xq_.data(), k_new, n, dim, heads, sp, rope_table_, context_len_, stream_));  // 1146, 1152 (new rows only)
       LCU_CHECK(lcu_attention(t_out_.data(), t_xq_.data(), kc, vc, n, T, sp, dim, heads, stream_));          // 1161-1171
     }
-    if (n == 1 && !fused_wo && dim <= 8192) {
+    if (n == 1 && hand_overs_ && !fused_wo && dim <= 8192) {
       // 1174 and 1176 in one launch (salts: even for this one, odd for the W2 launch below)
       LCU_CHECK(lcu_decode_proj_norm(x, t_norm_.data(), t_out_.data(), L.wo.data.data(), L.wo.scales.data(), block, dim,
                                      dim, L.ffn_norm.data(), p.norm_eps,
@@ -401,7 +408,7 @@ void llama_context_impl::enqueue_layers(int n) {
       matmul_multi(up_out, t_norm_.data(), up_w, 2, n);                                                      // 1180, 1181
       LCU_CHECK(lcu_silu_mul(t_silu_.data(), t_w1_.data(), t_w3_.data(), (size_t)n * ffn, stream_));         // 1183
     }
-    if (n == 1 && l + 1 < model_->layers.size() && dim <= 8192) {
+    if (n == 1 && hand_overs_ && l + 1 < model_->layers.size() && dim <= 8192) {
       // 1185 and the next layer's 1129 in one launch
       llama_layer const& next = model_->layers[l + 1];
       LCU_CHECK(lcu_decode_proj_norm(x, t_norm_.data(), t_silu_.data(), L.w2.data.data(), L.w2.scales.data(), block,
@@ -433,7 +440,9 @@ void llama_context_impl::enqueue_head(int n) {
                                 stream_));
   }
   // the first maximum of the fp16 probabilities is found on the device; 4 bytes go back to the host
-  LCU_CHECK(lcu_softmax_argmax(t_probs_.data(), t_argmax_.data(), t_logits_.data(), vocab, temperature_, stream_));
+  // and, next to it, the stream's count of hand-overs that did not arrive, for next_token's one copy back
+  LCU_CHECK(lcu_softmax_argmax_status(t_probs_.data(), t_argmax_.data(), t_logits_.data(), vocab, temperature_,
+                                      stream_));
   if (sampling_) {  // 1202-1203; the random bits of this step are in t_step_
     LCU_CHECK(lcu_sample_row(t_argmax_.data(), t_probs_.data(), vocab, 0,
                              (char*)t_step_.data() + offsetof(step_state, random), stream_));
@@ -560,17 +569,40 @@ short llama_context_impl::next_token(std::vector<short> const& new_tokens) {
   } else {
     enqueue_all();
   }
-  int token = 0;
-  LCU_CHECK(lcu_d2h(&token, t_argmax_.data(), sizeof(int), stream_));  // 1198-1200, blocks
-  // The one-token launches hand results over between their workgroups with bounded waits; a wait that
-  // ran out leaves a wrong result behind, which is a device error like any other: fatal.  Looked at
-  // every 32 steps (4 bytes back) and when the context goes away.
-  if (n == 1 && (decode_calls_ & 31) == 0) {
-    check_hand_overs();
+  struct {
+    int token;
+    unsigned timeouts;
+  } result{0, 0};
+  LCU_CHECK(lcu_d2h(&result, t_argmax_.data(), sizeof(result), stream_));  // 1198-1200, blocks
+  // The one-token launches hand results over between their workgroups with bounded waits, and a wait
+  // that ran out went on with stale words: the count of such waits comes back with the token, and a
+  // count that has moved means this step's token is not to be trusted.  It is never returned: the
+  // context leaves the hand-over launches for good (something else is holding compute units of this
+  // device), and the step is computed again by launches that wait for nobody -- the step is a function
+  // of the token, the position and the cache rows below the position, all untouched.
+  if (result.timeouts != timeouts_seen_) {
+    fprintf(stderr, "llama_context: %u hand-over(s) between workgroups of a decode launch did not arrive (is other "
+                    "work holding compute units of this device?); the step is recomputed without them\n",
+            result.timeouts - timeouts_seen_);
+    timeouts_seen_ = result.timeouts;
+    ++hand_over_fallbacks_;
+    if (!hand_overs_ || n != 1) {
+      // no launch of such a call hands anything over: somebody else is using this stream's workspace
+      fprintf(stderr, "llama_context: the count moved during a call that hands nothing over\n");
+      raise(SIGSEGV);
+    }
+    hand_overs_ = false;
+    drop_graph();
+    enqueue_all();
+    LCU_CHECK(lcu_d2h(&result, t_argmax_.data(), sizeof(result), stream_));
+    if (result.timeouts != timeouts_seen_) {
+      fprintf(stderr, "llama_context: the recomputed step reports hand-overs as well\n");
+      raise(SIGSEGV);
+    }
   }
   start_pos_ += n;
   last_n_ = n;
-  return (short)token;
+  return (short)result.token;
 }
 
 /* static */ std::unique_ptr<llama_context> llama_context::create(llama_model* model, int context_len,

@@ -66,6 +66,8 @@ struct llama_context_impl final : public llama_context {
   std::vector<kv_cache_layer>& kv() { return kv_; }
   void* rope_table() const { return rope_table_; }
   float temperature() const { return temperature_; }
+  // decode steps that were computed a second time because hand-overs inside a launch did not arrive
+  int hand_over_fallbacks() const { return hand_over_fallbacks_; }
   // a step taken for this sequence by llama_batch_context: one more cached row
   void advance_one() {
     start_pos_ += 1;
@@ -78,7 +80,6 @@ struct llama_context_impl final : public llama_context {
   void enqueue_layers(int n);
   void enqueue_head(int n);
   void drop_graph();
-  void check_hand_overs();
   std::vector<kv_cache_layer> kv_;
   gpu_buffer t_embed_, t_norm_, t_xq_, t_out_, t_w1_, t_w3_, t_silu_;
   gpu_buffer t_tokens_, t_logits_, t_probs_, t_argmax_;
@@ -101,6 +102,9 @@ struct llama_context_impl final : public llama_context {
   int decode_calls_{0};
   int decode_bound_{0};  // the position bound the decode graph was captured with
   int compute_units_{0};
+  bool hand_overs_{true};       // one-token steps use the launches that hand results over inside themselves
+  unsigned timeouts_seen_{0};   // the stream's count of hand-overs that did not arrive, as last read
+  int hand_over_fallbacks_{0};
   void* stream_{nullptr};
   void* rope_table_{nullptr};
   int last_n_{0};

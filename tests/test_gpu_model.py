@@ -393,6 +393,122 @@ def test_two_contexts_decoding_from_two_threads(gpu):
     gm.close()
 
 
+def test_decode_while_another_thread_prefills_and_steps_a_batch(gpu):
+    """One thread decodes with the launches that hand results over inside themselves while another thread keeps
+    the device busy with 512-token prompts and batched steps on streams of its own: the decoding thread must get
+    the tokens it gets alone (a hand-over that did not arrive in time would have its step recomputed, never
+    returned)."""
+    import threading
+    G = gpu
+    cfg = dict(dim=4096, multiple_of=256, n_heads=32, n_layers=2, n_vocab=512, norm_eps=1e-6, q_type=0, qblock=128)
+    gm = G.P.Model(**cfg, seed=5)
+    steps = 60
+    fallbacks = []
+
+    def decode(out):
+        c = G.P.Context(gm, context_len=128, temperature=0.8)
+        toks = [c.next_token([3, 7, 11, 200, 5])]
+        for _ in range(steps):
+            toks.append(c.next_token([toks[-1]]))
+        out.append(toks)
+        fallbacks.append(c.hand_over_fallbacks())
+        c.close()
+
+    alone = []
+    decode(alone)
+    stop = threading.Event()
+
+    def disturb():
+        rng = np.random.default_rng(1)
+        c = G.P.Context(gm, context_len=600, temperature=0.8)
+        bc = G.P.BatchContext(gm, 4, context_len=64, temperature=0.8)
+        for b in range(4):
+            bc.next_token(b, [5 + b, 9])
+        last = [1, 2, 3, 4]
+        while not stop.is_set():
+            c.clear_tokens()
+            c.next_token(rng.integers(0, cfg["n_vocab"], 512).astype(np.int16))
+            for b in range(4):
+                bc.clear_tokens(b)
+                bc.next_token(b, [5 + b, 9])
+            for _ in range(8):
+                last = bc.next_tokens(last)
+        bc.close()
+        c.close()
+
+    th = threading.Thread(target=disturb)
+    th.start()
+    together = []
+    try:
+        decode(together)
+    finally:
+        stop.set()
+        th.join()
+    assert together == alone
+    print("hand-over fallbacks alone / disturbed:", fallbacks)
+    gm.close()
+
+
+@pytest.mark.parametrize("q_type", [0, 1])
+def test_a_failed_hand_over_is_never_returned(gpu, q_type):
+    """The count of hand-overs that did not arrive comes back with every token.  Raised from the host between two
+    steps (no kernel is made to wait), it makes the next step take the path a real failure takes: the step's
+    first result is dropped, the context leaves the hand-over launches for good and computes the step again with
+    launches that wait for nobody -- same tokens and logits, to the bit, as an undisturbed context."""
+    G = gpu
+    L = G.B.lib()
+    cfg = dict(dim=4096, multiple_of=256, n_heads=32, n_layers=2, n_vocab=512, norm_eps=1e-6, q_type=q_type, qblock=128)
+    gm = G.P.Model(**cfg, seed=6)
+    prompt = [3, 7, 11, 200, 5, 17]
+
+    def run(inject_at):
+        c = G.P.Context(gm, context_len=64, temperature=0.8)
+        toks, logits = [c.next_token(prompt)], []
+        for k in range(12):
+            if k == inject_at:
+                G.B.check(L.lcu_sync_add_timeouts(c.stream, 3))
+            toks.append(c.next_token([toks[-1]]))
+            logits.append(c.logits().copy())
+        n = c.hand_over_fallbacks()
+        c.close()
+        return toks, logits, n
+
+    want, want_logits, n0 = run(None)
+    assert n0 == 0
+    # before the graph exists (step 0 runs eagerly, step 1 captures), on a replayed graph, and later
+    for at in (0, 1, 5):
+        got, got_logits, n = run(at)
+        assert n == 1, at
+        assert got == want, at
+        for a, b in zip(got_logits, want_logits):
+            assert (a.view(np.uint16) == b.view(np.uint16)).all(), at
+    gm.close()
+
+
+def test_contexts_without_hand_over_launches(gpu, monkeypatch):
+    """LLAMA_CU_NO_HANDOVER=1 (a device shared with other processes): one-token steps use launches whose
+    workgroups never wait for one another; same tokens and logits to the bit."""
+    G = gpu
+    cfg = dict(dim=4096, multiple_of=256, n_heads=32, n_layers=2, n_vocab=512, norm_eps=1e-6, q_type=0, qblock=128)
+    gm = G.P.Model(**cfg, seed=6)
+
+    def run():
+        c = G.P.Context(gm, context_len=64, temperature=0.8)
+        toks = [c.next_token([3, 7, 11, 200, 5, 17])]
+        for _ in range(8):
+            toks.append(c.next_token([toks[-1]]))
+        logits = c.logits().copy()
+        assert c.hand_over_fallbacks() == 0
+        c.close()
+        return toks, logits
+
+    want, want_logits = run()
+    monkeypatch.setenv("LLAMA_CU_NO_HANDOVER", "1")
+    got, got_logits = run()
+    assert got == want and (got_logits.view(np.uint16) == want_logits.view(np.uint16)).all()
+    gm.close()
+
+
 def test_context_length_limits(gpu):
     """The attention kernels bound the context length: a longer one is refused when the context is
     created (the reference leaves it free, llama_cu.h:376), never in the middle of a generation."""

@@ -197,6 +197,27 @@ def test_gemm_f16(gpu, M, K, N):
     G.release()
 
 
+def test_gemm_residual_into_an_output_that_is_not_16_byte_aligned(gpu):
+    """beta = 1 with the output tile 8 bytes off a 16-byte boundary: the tile that fetches its old values in 16-byte
+    pieces (512 x 4096 x 4096, the Wo product) must fall back to 2-byte reads; same bits as the aligned call."""
+    G = gpu
+    M, K, N = 512, 4096, 4096
+    x = normal((M, K), 0, 310, 1.0)
+    w = normal((N, K), 0, 311, 0.02)
+    old = normal((M, N), 0, 312, 1.0)
+    want = G.gemm_f16(x, w, beta=1.0, out=old)
+    buf = G.empty((M * N + 8,))
+    for shift in (4, 1):  # halves: 8 bytes and 2 bytes off
+        padded = np.zeros(M * N + 8, dtype=np.float16)
+        padded[shift:shift + M * N] = old.reshape(-1)
+        G.B.check(G.L().lcu_h2d(buf.ptr, padded.ctypes.data, padded.nbytes, None))
+        G.B.check(G.L().lcu_gemm_f16_nt(buf.ptr + 2 * shift, G.dev_keep(x).ptr, G.dev_keep(w).ptr, M, K, N, 1.0, None))
+        got = G.host(buf, (M * N + 8,))[shift:shift + M * N].reshape(M, N)
+        assert (got.view(np.uint16) == want.view(np.uint16)).all(), shift
+    buf.free()
+    G.release()
+
+
 def test_gemm_exact_cases(gpu):
     G = gpu
     K = 256

@@ -1,15 +1,20 @@
 """Writes the greedy-decoding fixtures under tests/golden/ with the CPU oracle.
 
-    python tests/golden/make_greedy_fixture.py llama7b_fp16 [seed]
-    python tests/golden/make_greedy_fixture.py llama30b_u8 [seed]
+    python tests/golden/make_greedy_fixture.py llama7b_fp16 [seed [prompt_len [steps [flavour]]]]
+    python tests/golden/make_greedy_fixture.py llama30b_u8 [seed [prompt_len [steps [flavour]]]]
 
 Each fixture holds the model shape, the seeds, the 512 prompt token ids, the 128 greedy tokens the
-oracle produces (matmul flavour 2: every sum in the order of the HIP kernels -- the matrix cores'
-steps of eight products and the dispatcher's cut of K for the prompt, the lane and wavefront order
-of the decode kernels, v_dot2_f32_f16 for uint8 weights -- so that the whole run can be held to the
-GPU bit for bit; temperature 0.8 as main.cpp:58), and for every step the two largest fp16 logits
-with their token ids and the two largest probabilities.  Only the oracle runs here; nothing from the reference is
-imported or executed.
+oracle produces (temperature 0.8 as main.cpp:58), and for every step the two largest fp16 logits
+with their token ids and the two largest probabilities.  Two fixtures per model:
+  flavour 2 (default) -> <name>_seed<seed>_greedy.json: every sum in the order of the HIP kernels
+    (the matrix cores' steps of eight products and the dispatcher's cut of K for the prompt, the
+    lane and wavefront order of the decode kernels, v_dot2_f32_f16 for uint8 weights), so that the
+    whole run can be held to the GPU bit for bit;
+  flavour 1 -> <name>_seed<seed>_greedy_reference_order.json: the sums as the reference's own
+    kernels order them (llama_cu.cu:150-366: 16-wide k steps per tile, sequential attention dots),
+    which is what ties the full-depth run to the reference's arithmetic; the GPU is held to it
+    within a tolerance, token for token except where the oracle's own two best logits nearly tie.
+Only the oracle runs here; nothing from the reference is imported or executed.
 """
 import json
 import os
@@ -35,11 +40,12 @@ def main():
     seed = int(sys.argv[2]) if len(sys.argv) > 2 else 0
     prompt_len = int(sys.argv[3]) if len(sys.argv) > 3 else 512
     steps = int(sys.argv[4]) if len(sys.argv) > 4 else 128
+    flavour = int(sys.argv[5]) if len(sys.argv) > 5 else 2
     cfg = CONFIGS[name]
     t0 = time.time()
     model = O.Model(norm_eps=1e-6, qblock=128, seed=seed, weight_std=0.02, **cfg)
     print("model built in %.1fs (ffn %d)" % (time.time() - t0, model.ffn), flush=True)
-    ctx = O.Context(model, context_len=2048, temperature=0.8, flavour=2)
+    ctx = O.Context(model, context_len=2048, temperature=0.8, flavour=flavour)
     prompt = np.random.default_rng(seed).integers(0, cfg["n_vocab"], prompt_len).astype(np.int16)
     tokens, top, top_ids = [], [], []
     feed = prompt
@@ -55,9 +61,9 @@ def main():
         top_ids.append([int(order[0]), int(order[1])])
         feed = np.array([tok], dtype=np.int16)
         print("step %d token %d logit margin %.5f (%.1fs)" % (step, tok, lo[1] - lo[0], time.time() - t1), flush=True)
-    out = dict(name=name, matmul_flavour=2, seed=seed, weight_std=0.02, norm_eps=1e-6, qblock=128, temperature=0.8, context_len=2048,
+    out = dict(name=name, matmul_flavour=flavour, seed=seed, weight_std=0.02, norm_eps=1e-6, qblock=128, temperature=0.8, context_len=2048,
                prompt=[int(t) for t in prompt], tokens=tokens, top2_logits_probs=top, top2_ids=top_ids, **cfg)
-    path = os.path.join(HERE, "%s_seed%d_greedy.json" % (name, seed))
+    path = os.path.join(HERE, "%s_seed%d_greedy%s.json" % (name, seed, "" if flavour == 2 else "_reference_order"))
     with open(path, "w") as f:
         json.dump(out, f)
     print("wrote", path, "in %.1fs" % (time.time() - t0))

@@ -691,19 +691,31 @@ def test_one_llama7b_layer_prefill_512_then_decode_at_2048(gpu):
 
 
 # Greedy decoding, teacher-forced (the oracle's token is fed back, so one differing step could not hide
-# the steps after it).  The fixtures come from the oracle's flavour 2, which restates the sums of every
-# kernel on the way -- the matrix cores' steps of eight products and the dispatcher's cut of K for the
-# 512-token prompt, the lane and wavefront order of the decode kernels, v_dot2_f32_f16 for uint8
-# weights -- so nothing is left to a tolerance: every step must give the oracle's token, and the two
-# largest logits the fixture records for a step must be the device's to the bit.
+# the steps after it), against two fixtures per model, both written by the CPU oracle:
+#  * kernel order (flavour 2), which restates the sums of every kernel on the way -- the matrix cores'
+#    steps of eight products and the dispatcher's cut of K for the 512-token prompt, the lane and
+#    wavefront order of the decode kernels, v_dot2_f32_f16 for uint8 weights -- so nothing is left to a
+#    tolerance: every step must give the oracle's token, and the two largest logits the fixture
+#    records for a step must be the device's to the bit;
+#  * reference order (flavour 1), the sums as the reference's own kernels order them: this is what ties
+#    the full-depth run to llama_cu.cu's arithmetic rather than to a restatement of this library.  Two
+#    orders of the same fp32 sums differ in the last bits and the difference grows through the layers,
+#    so here the bar is the tolerance: the two recorded logits within DEPTH_TOL of the device's
+#    (relative to the largest logit), and the same token at every step except where the oracle's own
+#    two best logits are closer than NEAR_TIE -- there the device may pick the other one of the two.
+#    NEAR_TIE is twice the largest logit deviation seen at that depth.
+DEPTH_TOL = {"llama7b_fp16": 1e-2, "llama30b_u8": 2e-2}
+NEAR_TIE = {"llama7b_fp16": 0.05, "llama30b_u8": 0.15}
 
 
-def greedy_case(G, name):
-    path = os.path.join(GOLDEN, name)
-    fx = json.load(open(path))
+def greedy_case(G, model_name):
+    fx = json.load(open(os.path.join(GOLDEN, model_name + "_seed0_greedy.json")))
+    fr = json.load(open(os.path.join(GOLDEN, model_name + "_seed0_greedy_reference_order.json")))
+    assert fx["matmul_flavour"] == 2 and fr["matmul_flavour"] == 1 and fx["prompt"] == fr["prompt"]
     gm = G.P.Model(dim=fx["dim"], multiple_of=fx["multiple_of"], n_heads=fx["n_heads"], n_layers=fx["n_layers"],
                    n_vocab=fx["n_vocab"], norm_eps=fx["norm_eps"], q_type=fx["q_type"], qblock=fx["qblock"],
                    seed=fx["seed"], weight_std=fx["weight_std"])
+    # kernel order: every bit
     gc = G.P.Context(gm, context_len=fx["context_len"], temperature=fx["temperature"])
     feed = np.array(fx["prompt"], dtype=np.int16)
     wrong_tokens, wrong_logits = [], []
@@ -717,23 +729,50 @@ def greedy_case(G, name):
         if got[i1] != l1 or got[i2] != l2:
             wrong_logits.append("step %d: device %.6f / %.6f, oracle %.6f / %.6f" % (step, got[i1], got[i2], l1, l2))
         feed = np.array([want], dtype=np.int16)
+    print("%s, kernel order: %d of %d tokens identical, top-2 logits identical on %d steps"
+          % (model_name, len(fx["tokens"]) - len(wrong_tokens), len(fx["tokens"]), len(fx["tokens"]) - len(wrong_logits)))
+    assert not wrong_tokens and not wrong_logits, "\n".join(wrong_tokens + wrong_logits)
+    assert gc.hand_over_fallbacks() == 0
+    # reference order: tolerance, and the same token away from the oracle's near ties
+    gc.clear_tokens()
+    feed = np.array(fr["prompt"], dtype=np.int16)
+    identical, near_ties, failures, worst_abs, worst_rel = 0, [], [], 0.0, 0.0
+    for step, want in enumerate(fr["tokens"]):
+        tok = gc.next_token(feed)
+        l1, l2, _, _ = fr["top2_logits_probs"][step]
+        got = gc.logits().astype(np.float64)
+        i1, i2 = fr["top2_ids"][step]
+        dev = max(abs(got[i1] - l1), abs(got[i2] - l2))
+        worst_abs = max(worst_abs, dev)
+        worst_rel = max(worst_rel, dev / np.max(np.abs(got)))
+        if tok == want:
+            identical += 1
+        elif l1 - l2 <= NEAR_TIE[model_name] and tok in (i1, i2):
+            near_ties.append("step %d: device %d, oracle %d; oracle top-2 logits %.5f / %.5f" % (step, tok, want, l1, l2))
+        else:
+            failures.append("step %d: device %d, oracle %d (top-2 ids %s); oracle top-2 logits %.5f / %.5f"
+                            % (step, tok, want, [i1, i2], l1, l2))
+        feed = np.array([want], dtype=np.int16)
     gc.close()
     gm.close()
-    print("%s: %d of %d tokens identical, top-2 logits identical on %d steps"
-          % (name, len(fx["tokens"]) - len(wrong_tokens), len(fx["tokens"]), len(fx["tokens"]) - len(wrong_logits)))
-    return wrong_tokens, wrong_logits
+    n_close = sum(1 for t in fr["top2_logits_probs"] if t[0] - t[1] <= NEAR_TIE[model_name])
+    print("%s, reference order: %d of %d tokens identical (%d steps of the oracle are near ties), near-tie steps taken "
+          "the other way: %s; largest deviation of a recorded logit %.4f (%.2e of the largest logit)"
+          % (model_name, identical, len(fr["tokens"]), n_close, near_ties or "none", worst_abs, worst_rel))
+    assert not failures, "\n".join(failures)
+    assert worst_rel <= DEPTH_TOL[model_name]
+    assert 2 * worst_abs <= NEAR_TIE[model_name]
 
 
 def test_greedy_tokens_llama7b_fp16(gpu):
-    """Full LLaMA-7B shape, fp16, 512-token prompt, 128 greedy steps: the oracle's tokens and logits."""
-    wrong_tokens, wrong_logits = greedy_case(gpu, "llama7b_fp16_seed0_greedy.json")
-    assert not wrong_tokens and not wrong_logits, "\n".join(wrong_tokens + wrong_logits)
+    """Full LLaMA-7B shape, fp16, 512-token prompt, 128 greedy steps: the kernel-order oracle's tokens and logits
+    to the bit, the reference-order oracle's within the tolerance."""
+    greedy_case(gpu, "llama7b_fp16")
 
 
 def test_greedy_tokens_llama30b_u8(gpu):
-    """LLaMA-30B shape, uint8 weights, 512-token prompt, 128 greedy steps: the oracle's tokens and logits."""
-    wrong_tokens, wrong_logits = greedy_case(gpu, "llama30b_u8_seed0_greedy.json")
-    assert not wrong_tokens and not wrong_logits, "\n".join(wrong_tokens + wrong_logits)
+    """LLaMA-30B shape, uint8 weights, 512-token prompt, 128 greedy steps, likewise."""
+    greedy_case(gpu, "llama30b_u8")
 
 
 def test_u8_and_f16_kernels_agree_at_30b_depth(gpu):

@@ -705,7 +705,7 @@ def test_one_llama7b_layer_prefill_512_then_decode_at_2048(gpu):
 #    two best logits are closer than NEAR_TIE -- there the device may pick the other one of the two.
 #    NEAR_TIE is twice the largest logit deviation seen at that depth.
 DEPTH_TOL = {"llama7b_fp16": 1e-2, "llama30b_u8": 2e-2}
-NEAR_TIE = {"llama7b_fp16": 0.05, "llama30b_u8": 0.15}
+NEAR_TIE = {"llama7b_fp16": 0.05, "llama30b_u8": 0.12}
 
 
 def greedy_case(G, model_name):

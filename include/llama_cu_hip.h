@@ -170,7 +170,10 @@ int lcu_sample_row(void* out_index_dev, const void* probs_dev, int n, uint64_t r
  * rotated) and v are the first T rows of a [*, dim] cache; causal: row r sees columns
  * c <= r + start_pos.  Scores are rounded to fp16, probabilities are rounded to fp16, the
  * weighted sum runs in fp32: the reference's three rounding points.  head_dim must be 128,
- * T <= 4096. */
+ * T <= 4096 (the multi-row kernel keeps a strip of 16 or 32 rows of scores in LDS).  A call with
+ * n_new == 1 hands scores over between workgroups inside its launch when `stream` was made by
+ * lcu_stream_create (such a stream owns its hand-over words); on the default stream and on streams
+ * made elsewhere, which share the device's, it takes launches that hand nothing over. */
 int lcu_attention(void* out_dev, const void* q_dev, const void* k_dev, const void* v_dev,
                   int n_new, int T, int start_pos, int dim, int n_heads, void* stream);
 

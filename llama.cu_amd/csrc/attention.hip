@@ -815,7 +815,8 @@ int launch_decode_attention(half_t* out, const half_t* q, const half_t* k, const
 // ---------------------------------------------------------------------------------------------
 constexpr int CW = 64;         // cache rows per staged chunk
 constexpr int QLD = HD + 8;    // LDS row stride (halves) of the Q and K tiles
-constexpr int MAX_T_PREFILL = 2048;
+constexpr int MAX_T_PREFILL = 4096;    // 16-row tiles: a strip of 16 x 4096 fp16 scores fits LDS; 32-row tiles reach 2048
+constexpr int MAX_T_PREFILL_32 = 2048;
 
 // BR: query rows per workgroup (16 or 32)
 // LDS row of position p of a V chunk (a permutation inside every block of 32 positions)
@@ -1084,7 +1085,7 @@ int lcu_attention(void* out_dev, const void* q_dev, const void* k_dev, const voi
   // and the rows are short (T <= 1024: 22 us against 29 us at n = T = 512, dim 4096); with long
   // rows the per-chunk overhead of the extra workgroups costs more than the balance gains.
   const long wgs32 = (long)((n_new + 31) / 32) * n_heads;
-  const int BR = (wgs32 < 1024 && T <= 1024) ? 16 : 32;
+  const int BR = ((wgs32 < 1024 && T <= 1024) || T > MAX_T_PREFILL_32) ? 16 : 32;
   const int n_tiles = (n_new + BR - 1) / BR;
   const int Tc_max = (T + CW - 1) / CW * CW;
   const size_t lds = prefill_lds_bytes(BR, Tc_max);
@@ -1095,7 +1096,7 @@ int lcu_attention(void* out_dev, const void* q_dev, const void* k_dev, const voi
     LCU_HIP(hipFuncSetAttribute((const void*)prefill_attention_kernel<16>, hipFuncAttributeMaxDynamicSharedMemorySize,
                                 (int)prefill_lds_bytes(16, MAX_T_PREFILL)));
     LCU_HIP(hipFuncSetAttribute((const void*)prefill_attention_kernel<32>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                (int)prefill_lds_bytes(32, MAX_T_PREFILL)));
+                                (int)prefill_lds_bytes(32, MAX_T_PREFILL_32)));
     attr_set[dev & 15] = true;
   }
   if (BR == 16) {

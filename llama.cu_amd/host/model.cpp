@@ -478,22 +478,6 @@ short llama_context_impl::next_token(std::vector<short> const& new_tokens) {
   const int n = (int)new_tokens.size();
   assert(n > 0);
   assert(new_tokens.size() + start_pos_ <= (size_t)context_len_);  // llama_cu.cu:1074
-  if (n > 1 && start_pos_ + n > LLAMA_CU_MAX_PREFILL_ROWS) {
-    // The multi-row attention kernel covers cache rows up to LLAMA_CU_MAX_PREFILL_ROWS: what fits
-    // below that goes in one call, every later token as a call of its own (same results: a row
-    // of a multi-row call and a one-row call compute the same thing, llama_cu.cu:1099-1186).
-    size_t done = 0;
-    short last = 0;
-    if (start_pos_ + 1 < LLAMA_CU_MAX_PREFILL_ROWS) {
-      done = (size_t)(LLAMA_CU_MAX_PREFILL_ROWS - start_pos_);
-      last = next_token(std::vector<short>(new_tokens.begin(), new_tokens.begin() + done));
-    }
-    for (; done < new_tokens.size(); ++done) {
-      last = next_token(std::vector<short>(1, new_tokens[done]));
-    }
-    last_n_ = 1;
-    return last;
-  }
   const int dim = p.dim, vocab = p.n_vocab;
   const int block = p.q_type == quantization_type::uint8 ? p.quantization_block_size : 0;
   char* x = (char*)t_embed_.data();

@@ -8,10 +8,9 @@
 
 namespace llama_cu {
 
-// limits of the attention kernels (csrc/attention.hip): cache rows a one-token call can attend to,
-// and cache rows a multi-token call can
+// limit of the attention kernels (csrc/attention.hip): cache rows a call can attend to, whether it
+// brings one new token or many
 constexpr int LLAMA_CU_MAX_CONTEXT = 4096;
-constexpr int LLAMA_CU_MAX_PREFILL_ROWS = 2048;
 
 
 // one weight matrix [rows, cols]: fp16 values, or uint8 codes with fp16 scales [rows, cols/block]

@@ -547,7 +547,7 @@ def test_memset_and_copies(gpu):
 
 
 ATT_CASES = [(1, 1), (1, 2), (1, 255), (1, 256), (1, 257), (1, 577), (1, 2048), (5, 5), (64, 64), (70, 70),
-             (512, 512), (3, 130), (40, 300)]
+             (512, 512), (3, 130), (40, 300), (300, 2100), (64, 4096), (1, 4096)]
 
 
 @pytest.mark.parametrize("n,T", ATT_CASES)

@@ -5,7 +5,8 @@ import os
 import numpy as np
 
 _PKG = os.path.dirname(os.path.abspath(__file__))
-_LIB_PATH = os.path.join(_PKG, "libllama_cu_amd.so")
+# LLAMA_CU_AMD_LIB names another build of the same library (the diagnostic one of build.py --timeline)
+_LIB_PATH = os.environ.get("LLAMA_CU_AMD_LIB") or os.path.join(_PKG, "libllama_cu_amd.so")
 _lib = None
 
 

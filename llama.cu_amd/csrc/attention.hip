@@ -444,6 +444,27 @@ __global__ __launch_bounds__(256) void decode_attention_spread_kernel(
 // four wavefronts as gemv_kernel<false, 1 or 2, 2, 0> does it (chunk c of 512 elements to
 // wavefront (c / 2) % 4, two accumulators per lane, wave_sum, wavefronts in order, then
 // fmaf(1, x, sum)), the norm by 256 threads as rmsnorm_kernel.  NB: dim <= 4096 * NB.
+// ---- phase timeline of the fused launch (diagnostic builds only: -DLCU_PHASE_TIMELINE) ------------
+// Thread 0 of every workgroup (and the first lane of its first Wo wavefront) notes the 100 MHz
+// real-time counter at the ends of the launch's phases into a device array, one row per launch (by
+// salt) and workgroup; lcu_debug_timeline_read copies it out.  Nothing of this exists in the
+// ordinary build.
+#ifdef LCU_PHASE_TIMELINE
+constexpr int TL_POINTS = 16, TL_LAUNCHES = 64, TL_GROUPS = 512;
+static __device__ uint64_t phase_timeline[TL_LAUNCHES * TL_GROUPS * TL_POINTS];
+#define TL_MARK(point)                                                                                          \
+  do {                                                                                                          \
+    if (threadIdx.x == ((point) >= 12 ? 256 : 0)) {                                                             \
+      phase_timeline[((tl_launch & (TL_LAUNCHES - 1)) * TL_GROUPS + blockIdx.x) * TL_POINTS + (point)] =        \
+          __builtin_amdgcn_s_memrealtime();                                                                     \
+    }                                                                                                           \
+  } while (0)
+#else
+#define TL_MARK(point) \
+  do {                 \
+  } while (0)
+#endif
+
 constexpr int FUSED_THREADS = 1024;
 constexpr int FUSED_PAD_LDS = 72 << 10;  // dynamic LDS nobody touches: a second workgroup does not fit the compute unit
 
@@ -505,6 +526,10 @@ __global__ __launch_bounds__(FUSED_THREADS) void decode_attention_wo_norm_kernel
   const bool att = tid < 256;
   int T = T_cap;
   if (pos_dev) T = min(max(*pos_dev + 1, 1), T_cap);
+#ifdef LCU_PHASE_TIMELINE
+  const uint32_t tl_launch = epoch;  // the salt: the layer
+#endif
+  TL_MARK(0);
   if (seq_dev) epoch = (epoch | (*seq_dev << 10)) & 0x7fffffffu;
   uint64_t* srow = exch + (size_t)h * T_cap;
   // what the 16 finishing threads need from memory at the very end, requested now
@@ -580,6 +605,7 @@ __global__ __launch_bounds__(FUSED_THREADS) void decode_attention_wo_norm_kernel
         __hip_atomic_store(srow + p, word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       }
     }
+    TL_MARK(1);
     uint64_t raw[NJ];
     int spins = 0;
     while (true) {
@@ -604,6 +630,7 @@ __global__ __launch_bounds__(FUSED_THREADS) void decode_attention_wo_norm_kernel
       }
       __builtin_amdgcn_s_sleep(1);
     }
+    TL_MARK(2);
 #pragma unroll
     for (int j = 0; j < NJ; ++j) x[j] = (float)__builtin_bit_cast(half_t, (unsigned short)raw[j]);
     m = x[0];
@@ -613,6 +640,7 @@ __global__ __launch_bounds__(FUSED_THREADS) void decode_attention_wo_norm_kernel
     if (lane == 0) red[wave] = m;
   }
   __syncthreads();  // (1)
+  TL_MARK(3);
 
   load_wo(B0, B1);
 
@@ -643,7 +671,9 @@ __global__ __launch_bounds__(FUSED_THREADS) void decode_attention_wo_norm_kernel
   load_wo(B1, B2);
   if (att && (tid & 31) == 0) red[tid >> 5] = ssum;
   __syncthreads();  // (3)
+  TL_MARK(4);
   load_wo(B2, LOADS);
+  TL_MARK(12);
   if (att) {
     const float4_t lo = *reinterpret_cast<const float4_t*>(red), hi = *reinterpret_cast<const float4_t*>(red + 4);
     const float total = ((lo[0] + hi[0]) + (lo[2] + hi[2])) + ((lo[1] + hi[1]) + (lo[3] + hi[3]));
@@ -653,6 +683,7 @@ __global__ __launch_bounds__(FUSED_THREADS) void decode_attention_wo_norm_kernel
     }
   }
   __syncthreads();  // (4)
+  TL_MARK(5);
   if (att) {
     float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
@@ -674,10 +705,12 @@ __global__ __launch_bounds__(FUSED_THREADS) void decode_attention_wo_norm_kernel
     for (int g = 0; g < 64; ++g) o += gsum[g][tid];
     publish16(exch + EXCH_ATT, row0, round_f16(o), epoch);  // 529
   }
+  TL_MARK(6);
 
   // ---- x + Wo . att for the 16 rows (llama_cu.cu:1174)
   gather_row(xs, exch + EXCH_ATT, dim, epoch, timeouts);
   __syncthreads();  // (6)
+  TL_MARK(7);
   if (team > 0) {
     half8_t xp[NB][2];  // this lane's pieces of the attention output, the same for every row
 #pragma unroll
@@ -712,7 +745,9 @@ __global__ __launch_bounds__(FUSED_THREADS) void decode_attention_wo_norm_kernel
       if (lane == 0 && r < 16) part[r][tw] = s;
     }
   }
+  TL_MARK(13);
   __syncthreads();  // (7) also: every read of the attention output in xs is done
+  TL_MARK(8);
   if (tid < 16) {
     float acc = 0.0f;
 #pragma unroll
@@ -721,11 +756,13 @@ __global__ __launch_bounds__(FUSED_THREADS) void decode_attention_wo_norm_kernel
     x_io[row0 + tid] = xn;
     publish16(exch + EXCH_X, row0, xn, epoch);
   }
+  TL_MARK(9);
 
   // ---- rms_norm of the new row (llama_cu.cu:1176, 66-107): every workgroup sums the squares, each
   // normalises its own 16 elements
   gather_row(xs, exch + EXCH_X, dim, epoch, timeouts);
   __syncthreads();  // (8)
+  TL_MARK(10);
   float sq = 0.0f;
   if (att) {
     // eight LDS reads in flight at a time; the additions stay in ascending order
@@ -761,6 +798,7 @@ __global__ __launch_bounds__(FUSED_THREADS) void decode_attention_wo_norm_kernel
     const half_t inner = round_f16((float)xs[row0 + tid] * rms_inv);
     norm_out[row0 + tid] = round_f16((float)nw_mine * (float)inner);
   }
+  TL_MARK(11);
 }
 
 // seq_dev == nullptr: the epoch is a number the host draws per launch (never under stream capture:
@@ -1222,5 +1260,22 @@ int lcu_attention_decode_batch(void* out_dev, const void* q_dev, const void* k_c
   LCU_LAUNCH_CHECK();
   return LCU_OK;
 }
+
+#ifdef LCU_PHASE_TIMELINE
+// diagnostic builds only: clears (out_host == NULL) or copies out the phase timeline of
+// lcu_decode_attention_wo_norm, uint64[64 launches][512 workgroups][16 points] of the 100 MHz counter
+int lcu_debug_timeline_read(void* out_host, size_t bytes) {
+  void* dev = nullptr;
+  LCU_HIP(hipGetSymbolAddress(&dev, HIP_SYMBOL(phase_timeline)));
+  LCU_HIP(hipDeviceSynchronize());
+  if (out_host == nullptr) {
+    LCU_HIP(hipMemset(dev, 0, sizeof(uint64_t) * TL_LAUNCHES * TL_GROUPS * TL_POINTS));
+  } else {
+    LCU_REQUIRE(bytes <= sizeof(uint64_t) * TL_LAUNCHES * TL_GROUPS * TL_POINTS, "lcu_debug_timeline_read: too many bytes");
+    LCU_HIP(hipMemcpy(out_host, dev, bytes, hipMemcpyDeviceToHost));
+  }
+  return LCU_OK;
+}
+#endif
 
 }  // extern "C"

@@ -236,7 +236,7 @@ struct batch_t {
 // wavefront w covers chunks (b * WAVES + w) * U .. + U.  begin() requests the first batch (weights,
 // x, norm weights); the caller may then reduce the norm statistics; run() does the rest and ends
 // with the cross-wavefront sum.
-template <bool U8, int R, int U, bool NORM, class Tasks>
+template <bool U8, int R, int U, bool NORM, class Tasks, int NB = 0>
 struct stream_t {
   using batch = batch_t<U8, R, U, NORM>;
   const Tasks tk;  // by value: a reference member kept the struct in scratch memory in some instantiations
@@ -245,7 +245,7 @@ struct stream_t {
   int K, block, block_shift, lane, wave, task, n_batches;
   const uint8_t* rows[R];
   const half_t* srow[R];
-  batch cur;
+  batch held[NB > 0 ? NB : 1];  // NB > 0: every batch of the rows (n_batches <= NB), all requested by begin()
 
   __device__ __forceinline__ stream_t(const Tasks& t, const half_t* x_, const half_t* norm_w_, int K_, int block_,
                                       int task_)
@@ -256,7 +256,10 @@ struct stream_t {
 
   __device__ __forceinline__ void begin() {
     tk.rows(task, rows, srow);
-    cur.load(rows, srow, x, norm_w, wave, K, block, block_shift, lane);
+#pragma unroll
+    for (int b = 0; b < (NB > 0 ? NB : 1); ++b) {
+      held[b].load(rows, srow, x, norm_w, b * GEMV_WAVES + wave, K, block, block_shift, lane);
+    }
   }
 
   // xs: raw x in LDS when NORM; part: GEMV_WAVES * R floats of LDS
@@ -267,13 +270,20 @@ struct stream_t {
       a0[r] = 0.0f;
       a1[r] = 0.0f;
     }
-    for (int b = 0; b < n_batches; ++b) {
-      batch nxt;
-      if (b + 1 < n_batches) {
-        nxt.load(rows, srow, x, norm_w, (b + 1) * GEMV_WAVES + wave, K, block, block_shift, lane);
+    if constexpr (NB > 0) {
+#pragma unroll
+      for (int b = 0; b < NB; ++b) {
+        held[b].fma(xs, rms_inv, b * GEMV_WAVES + wave, K, lane, a0, a1);
       }
-      cur.fma(xs, rms_inv, b * GEMV_WAVES + wave, K, lane, a0, a1);
-      cur = nxt;
+    } else {
+      for (int b = 0; b < n_batches; ++b) {
+        batch nxt;
+        if (b + 1 < n_batches) {
+          nxt.load(rows, srow, x, norm_w, (b + 1) * GEMV_WAVES + wave, K, block, block_shift, lane);
+        }
+        held[0].fma(xs, rms_inv, b * GEMV_WAVES + wave, K, lane, a0, a1);
+        held[0] = nxt;
+      }
     }
 #pragma unroll
     for (int r = 0; r < R; ++r) {
@@ -444,7 +454,7 @@ struct ffn_up_tasks {
 // ---- kernels -------------------------------------------------------------------------------------
 // one workgroup per task (blockIdx.x)
 // XN > 0: x is RMS-normalised first, from XN 16-byte pieces per thread (x_stage_t)
-template <bool U8, int R, int U, int XN>
+template <bool U8, int R, int U, int XN, int NB = 0>
 __global__ __launch_bounds__(GEMV_THREADS) void gemv_kernel(half_t* __restrict__ out, const half_t* __restrict__ x,
                                                             const half_t* __restrict__ norm_w, const void* __restrict__ W,
                                                             const half_t* __restrict__ S, int K, int N, int block,
@@ -454,7 +464,7 @@ __global__ __launch_bounds__(GEMV_THREADS) void gemv_kernel(half_t* __restrict__
   __shared__ float part[GEMV_WAVES * R];
   constexpr bool NORM = XN > 0;
   plain_tasks<U8, R> tk{W, S, out, K, N, U8 ? K / block : 0, beta};
-  stream_t<U8, R, U, NORM, plain_tasks<U8, R>> st(tk, x, norm_w, K, block, blockIdx.x);
+  stream_t<U8, R, U, NORM, plain_tasks<U8, R>, NB> st(tk, x, norm_w, K, block, blockIdx.x);
   float rms_inv = 1.0f;
   if constexpr (NORM) {
     x_stage_t<XN> xp;
@@ -469,7 +479,7 @@ __global__ __launch_bounds__(GEMV_THREADS) void gemv_kernel(half_t* __restrict__
   st.run(xs, rms_inv, part);
 }
 
-template <bool U8, int U, int XN, int PAIRS>
+template <bool U8, int U, int XN, int PAIRS, int NB = 0>
 __global__ __launch_bounds__(GEMV_THREADS) void decode_qkv_kernel(
     half_t* __restrict__ q_out, half_t* __restrict__ k_row, half_t* __restrict__ v_row, const half_t* __restrict__ x,
     const half_t* __restrict__ norm_w, const void* __restrict__ wq, const void* __restrict__ wk,
@@ -495,7 +505,7 @@ __global__ __launch_bounds__(GEMV_THREADS) void decode_qkv_kernel(
   qkv_tasks<U8, PAIRS> tk{W, S, dst, which == 2 ? nullptr : rope_row, dim, head_dim, U8 ? dim / block : 0,
                           which * tasks_per_matrix};
   constexpr bool NORM = XN > 0;
-  stream_t<U8, 2 * PAIRS, U, NORM, qkv_tasks<U8, PAIRS>> st(tk, x, norm_w, dim, block, blockIdx.x);
+  stream_t<U8, 2 * PAIRS, U, NORM, qkv_tasks<U8, PAIRS>, NB> st(tk, x, norm_w, dim, block, blockIdx.x);
   float rms_inv = 1.0f;
   if constexpr (NORM) {
     x_stage_t<XN> xp;
@@ -510,7 +520,7 @@ __global__ __launch_bounds__(GEMV_THREADS) void decode_qkv_kernel(
   st.run(xs, rms_inv, part);
 }
 
-template <bool U8, int U, int XN, int PAIRS>
+template <bool U8, int U, int XN, int PAIRS, int NB = 0>
 __global__ __launch_bounds__(GEMV_THREADS) void decode_ffn_up_kernel(
     half_t* __restrict__ out, const half_t* __restrict__ x, const half_t* __restrict__ norm_w,
     const void* __restrict__ w1, const void* __restrict__ w3, const half_t* __restrict__ s1,
@@ -520,7 +530,7 @@ __global__ __launch_bounds__(GEMV_THREADS) void decode_ffn_up_kernel(
   __shared__ float part[GEMV_WAVES * 2 * PAIRS];
   ffn_up_tasks<U8, PAIRS> tk{w1, w3, s1, s3, out, dim, U8 ? dim / block : 0, ffn};
   constexpr bool NORM = XN > 0;
-  stream_t<U8, 2 * PAIRS, U, NORM, ffn_up_tasks<U8, PAIRS>> st(tk, x, norm_w, dim, block, blockIdx.x);
+  stream_t<U8, 2 * PAIRS, U, NORM, ffn_up_tasks<U8, PAIRS>, NB> st(tk, x, norm_w, dim, block, blockIdx.x);
   float rms_inv = 1.0f;
   if constexpr (NORM) {
     x_stage_t<XN> xp;
@@ -545,7 +555,7 @@ __global__ __launch_bounds__(GEMV_THREADS) void decode_ffn_up_kernel(
 constexpr int FOLLOW_SPIN_LIMIT = 1 << 16;
 constexpr int FOLLOW_PIECES = 8;  // 16-byte requests per thread: N <= 8192
 
-template <bool U8, int R, int U>
+template <bool U8, int R, int U, int NB = 0>
 __global__ __launch_bounds__(GEMV_THREADS) void decode_proj_norm_kernel(
     half_t* __restrict__ x_io, half_t* __restrict__ norm_out, const half_t* __restrict__ lhs,
     const void* __restrict__ W, const half_t* __restrict__ S, const half_t* __restrict__ norm_w, int K, int N, int block,
@@ -558,7 +568,7 @@ __global__ __launch_bounds__(GEMV_THREADS) void decode_proj_norm_kernel(
   const int n_tasks = (N + R - 1) / R;
   if ((int)blockIdx.x < n_tasks) {
     proj_norm_tasks<U8, R> tk{W, S, x_io, words, K, N, U8 ? K / block : 0, epoch};
-    stream_t<U8, R, U, false, proj_norm_tasks<U8, R>> st(tk, lhs, nullptr, K, block, blockIdx.x);
+    stream_t<U8, R, U, false, proj_norm_tasks<U8, R>, NB> st(tk, lhs, nullptr, K, block, blockIdx.x);
     st.begin();
     st.run(xs, 1.0f, part);
     return;
@@ -656,6 +666,43 @@ void with_x_pieces(int dim, F&& f) {
   }
 }
 
+// uint8 rows at U = 1: a batch of the workgroup covers 4096 codes of a row.  Rows of two to five
+// batches have every batch requested at once (NB: same chunks on the same wavefronts in the same
+// order as the loop, so the same sums), longer ones keep the loop (NB = 0): 6656 x 17920 uint8
+// 23.6 -> 22.0 us, 5120 x 13824 15.5 -> 14.2, 4096 x 11008 10.9 -> 10.2, 8192^2 13.8 -> 13.3,
+// 17920 x 6656 20.8 -> 20.5, variants alternating in one process.  (fp16 rows gain at some lengths
+// and lose at others, 4096 x 11008 16.6 against 16.1 us, and keep the loop.)
+template <class F>
+void with_u8_batches(int K, F&& f) {
+  const int nb = (K + 4095) / 4096;
+  switch (nb) {
+    case 2: f(std::integral_constant<int, 2>{}); break;
+    case 3: f(std::integral_constant<int, 3>{}); break;
+    case 4: f(std::integral_constant<int, 4>{}); break;
+    case 5: f(std::integral_constant<int, 5>{}); break;
+    default: f(std::integral_constant<int, 0>{}); break;
+  }
+}
+
+// with_x_pieces and with_u8_batches for a row of dim codes: f(pieces of x per thread, NB)
+template <class F>
+void with_u8_row_plan(int dim, F&& f) {
+  using std::integral_constant;
+  if (dim <= 4096) {
+    f(integral_constant<int, 2>{}, integral_constant<int, 0>{});
+  } else if (dim <= 8192) {
+    f(integral_constant<int, 4>{}, integral_constant<int, 2>{});
+  } else if (dim <= 12288) {
+    f(integral_constant<int, 12>{}, integral_constant<int, 3>{});
+  } else if (dim <= 16384) {
+    f(integral_constant<int, 12>{}, integral_constant<int, 4>{});
+  } else if (dim <= 20480) {
+    f(integral_constant<int, 12>{}, integral_constant<int, 5>{});
+  } else {
+    f(integral_constant<int, 12>{}, integral_constant<int, 0>{});
+  }
+}
+
 int check_quant_args(const char* who, const void* scales, int K, int block) {
   LCU_REQUIRE(scales != nullptr, "%s: quantised weights need scales", who);
   LCU_REQUIRE(block >= 16 && block % 16 == 0 && K % block == 0 && K % 16 == 0,
@@ -683,11 +730,15 @@ int gemv_u8(half_t* out, const half_t* x, const uint8_t* W, const half_t* S, int
   // four rows per workgroup where that still gives most compute units eight workgroups: x (as many
   // bytes as two rows of codes) is then fetched half as often (30B shapes: W1/W3 41.5 -> 38.9 us,
   // the logits 216 MB in 34 us); at N = 4096 it would leave half the workgroup slots empty
-  if (N >= 6144) {
-    gemv_kernel<true, 4, 1, 0><<<(N + 3) / 4, GEMV_THREADS, 0, st>>>(out, x, nullptr, W, S, K, N, block, beta, 0.f);
-  } else {
-    gemv_kernel<true, 2, 1, 0><<<(N + 1) / 2, GEMV_THREADS, 0, st>>>(out, x, nullptr, W, S, K, N, block, beta, 0.f);
-  }
+  with_u8_batches(K, [&](auto nb) {
+    if (N >= 6144) {
+      gemv_kernel<true, 4, 1, 0, decltype(nb)::value><<<(N + 3) / 4, GEMV_THREADS, 0, st>>>(out, x, nullptr, W, S, K, N,
+                                                                                          block, beta, 0.f);
+    } else {
+      gemv_kernel<true, 2, 1, 0, decltype(nb)::value><<<(N + 1) / 2, GEMV_THREADS, 0, st>>>(out, x, nullptr, W, S, K, N,
+                                                                                          block, beta, 0.f);
+    }
+  });
   LCU_LAUNCH_CHECK();
   return LCU_OK;
 }
@@ -723,17 +774,20 @@ int lcu_decode_qkv(void* q_out_dev, void* k_cache_dev, void* v_cache_dev, const 
     if (rc) return rc;
     LCU_REQUIRE(sk_dev && sv_dev, "lcu_decode_qkv: quantised weights need scales");
     if (norm_w_dev) {
-      with_x_pieces(dim, [&](auto xn) {
-        decode_qkv_kernel<true, 1, decltype(xn)::value, 1><<<grid, GEMV_THREADS, decltype(xn)::value * 4096, st>>>(
+      with_u8_row_plan(dim, [&](auto xn, auto nb) {
+        decode_qkv_kernel<true, 1, decltype(xn)::value, 1, decltype(nb)::value>
+            <<<grid, GEMV_THREADS, decltype(xn)::value * 4096, st>>>(
             (half_t*)q_out_dev, k_row, v_row, (const half_t*)x_dev, (const half_t*)norm_w_dev, wq_dev, wk_dev, wv_dev,
             (const half_t*)sq_dev, (const half_t*)sk_dev, (const half_t*)sv_dev, block, dim, head_dim, eps, rope_row,
             (const int*)pos_dev, table_positions - 1);
       });
     } else {
-      decode_qkv_kernel<true, 1, 0, 2><<<grid / 2, GEMV_THREADS, 0, st>>>(
-          (half_t*)q_out_dev, k_row, v_row, (const half_t*)x_dev, nullptr, wq_dev, wk_dev, wv_dev,
-          (const half_t*)sq_dev, (const half_t*)sk_dev, (const half_t*)sv_dev, block, dim, head_dim, eps, rope_row, (const int*)pos_dev,
-          table_positions - 1);
+      with_u8_batches(dim, [&](auto nb) {
+        decode_qkv_kernel<true, 1, 0, 2, decltype(nb)::value><<<grid / 2, GEMV_THREADS, 0, st>>>(
+            (half_t*)q_out_dev, k_row, v_row, (const half_t*)x_dev, nullptr, wq_dev, wk_dev, wv_dev,
+            (const half_t*)sq_dev, (const half_t*)sk_dev, (const half_t*)sv_dev, block, dim, head_dim, eps, rope_row,
+            (const int*)pos_dev, table_positions - 1);
+      });
     }
   } else {
     if (norm_w_dev) {
@@ -770,15 +824,17 @@ int lcu_decode_proj_norm(void* x_io_dev, void* norm_out_dev, const void* lhs_dev
     if (rc) return rc;
     // four rows per workgroup (x fetched half as often) where the rows are long; short rows (Wo) finish sooner
     // as twice as many workgroups of two
-    if (N >= 6144 && K >= 8192) {
-      decode_proj_norm_kernel<true, 4, 1><<<(N + 3) / 4 + 1, GEMV_THREADS, lds, st>>>(
-          (half_t*)x_io_dev, (half_t*)norm_out_dev, (const half_t*)lhs_dev, w_dev, (const half_t*)scales_dev,
-          (const half_t*)norm_w_dev, K, N, block, eps, words, (const uint32_t*)seq_dev, (uint32_t)salt, timeouts);
-    } else {
-      decode_proj_norm_kernel<true, 2, 1><<<(N + 1) / 2 + 1, GEMV_THREADS, lds, st>>>(
-          (half_t*)x_io_dev, (half_t*)norm_out_dev, (const half_t*)lhs_dev, w_dev, (const half_t*)scales_dev,
-          (const half_t*)norm_w_dev, K, N, block, eps, words, (const uint32_t*)seq_dev, (uint32_t)salt, timeouts);
-    }
+    with_u8_batches(K, [&](auto nb) {
+      if (N >= 6144 && K >= 8192) {
+        decode_proj_norm_kernel<true, 4, 1, decltype(nb)::value><<<(N + 3) / 4 + 1, GEMV_THREADS, lds, st>>>(
+            (half_t*)x_io_dev, (half_t*)norm_out_dev, (const half_t*)lhs_dev, w_dev, (const half_t*)scales_dev,
+            (const half_t*)norm_w_dev, K, N, block, eps, words, (const uint32_t*)seq_dev, (uint32_t)salt, timeouts);
+      } else {
+        decode_proj_norm_kernel<true, 2, 1, decltype(nb)::value><<<(N + 1) / 2 + 1, GEMV_THREADS, lds, st>>>(
+            (half_t*)x_io_dev, (half_t*)norm_out_dev, (const half_t*)lhs_dev, w_dev, (const half_t*)scales_dev,
+            (const half_t*)norm_w_dev, K, N, block, eps, words, (const uint32_t*)seq_dev, (uint32_t)salt, timeouts);
+      }
+    });
   } else {
     decode_proj_norm_kernel<false, 2, 2><<<(N + 1) / 2 + 1, GEMV_THREADS, lds, st>>>(
         (half_t*)x_io_dev, (half_t*)norm_out_dev, (const half_t*)lhs_dev, w_dev, nullptr, (const half_t*)norm_w_dev, K, N,
@@ -801,15 +857,18 @@ int lcu_decode_ffn_up(void* out_dev, const void* x_dev, const void* norm_w_dev, 
     if (rc) return rc;
     LCU_REQUIRE(s3_dev != nullptr, "lcu_decode_ffn_up: quantised weights need scales");
     if (norm_w_dev) {
-      with_x_pieces(dim, [&](auto xn) {
-        decode_ffn_up_kernel<true, 1, decltype(xn)::value, 1><<<grid, GEMV_THREADS, decltype(xn)::value * 4096, st>>>(
+      with_u8_row_plan(dim, [&](auto xn, auto nb) {
+        decode_ffn_up_kernel<true, 1, decltype(xn)::value, 1, decltype(nb)::value>
+            <<<grid, GEMV_THREADS, decltype(xn)::value * 4096, st>>>(
             (half_t*)out_dev, (const half_t*)x_dev, (const half_t*)norm_w_dev, w1_dev, w3_dev, (const half_t*)s1_dev,
             (const half_t*)s3_dev, block, dim, ffn, eps);
       });
     } else {
-      decode_ffn_up_kernel<true, 1, 0, 2><<<(grid + 1) / 2, GEMV_THREADS, 0, st>>>(
-          (half_t*)out_dev, (const half_t*)x_dev, nullptr, w1_dev, w3_dev, (const half_t*)s1_dev,
-          (const half_t*)s3_dev, block, dim, ffn, eps);
+      with_u8_batches(dim, [&](auto nb) {
+        decode_ffn_up_kernel<true, 1, 0, 2, decltype(nb)::value><<<(grid + 1) / 2, GEMV_THREADS, 0, st>>>(
+            (half_t*)out_dev, (const half_t*)x_dev, nullptr, w1_dev, w3_dev, (const half_t*)s1_dev,
+            (const half_t*)s3_dev, block, dim, ffn, eps);
+      });
     }
   } else {
     if (norm_w_dev) {
@@ -837,8 +896,9 @@ int lcu_decode_logits(void* logits_dev, const void* x_dev, const void* norm_w_de
   if (block > 0) {
     int rc = check_quant_args("lcu_decode_logits", sout_dev, dim, block);
     if (rc) return rc;
-    with_x_pieces(dim, [&](auto xn) {
-      gemv_kernel<true, 2, 1, decltype(xn)::value><<<grid, GEMV_THREADS, decltype(xn)::value * 4096, st>>>(
+    with_u8_row_plan(dim, [&](auto xn, auto nb) {
+      gemv_kernel<true, 2, 1, decltype(xn)::value, decltype(nb)::value>
+          <<<grid, GEMV_THREADS, decltype(xn)::value * 4096, st>>>(
           (half_t*)logits_dev, (const half_t*)x_dev, (const half_t*)norm_w_dev, wout_dev, (const half_t*)sout_dev, dim,
           n_vocab, block, 0.0f, eps);
     });

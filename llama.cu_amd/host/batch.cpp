@@ -16,6 +16,7 @@ struct llama_batch_context_impl final : public llama_batch_context {
   llama_batch_context_impl(llama_model* model, int n_sequences, int context_len, float temperature)
       : model_(static_cast<llama_model_impl*>(model)), context_len_(context_len), temperature_(temperature) {
     LCU_CHECK(lcu_init(0));
+    device_structure_lock lock(device_structure_mutex());
     LCU_CHECK(lcu_stream_create(&stream_));
     for (int b = 0; b < n_sequences; ++b) {
       seqs_.push_back(std::make_unique<llama_context_impl>(model, context_len, temperature));
@@ -41,6 +42,7 @@ struct llama_batch_context_impl final : public llama_batch_context {
 
   ~llama_batch_context_impl() override {
     lcu_sync(stream_);
+    device_structure_lock lock(device_structure_mutex());
     lcu_graph_destroy(graph_);
     lcu_stream_destroy(stream_);
   }
@@ -96,15 +98,18 @@ struct llama_batch_context_impl final : public llama_batch_context {
     }
     graph_bound_ = bound;
     ++calls_;
-    if (!graph_ && calls_ >= 2) {
-      LCU_CHECK(lcu_graph_begin_capture(stream_));
-      enqueue_step(bound);
-      LCU_CHECK(lcu_graph_end_capture(stream_, &graph_));
-    }
-    if (graph_) {
-      LCU_CHECK(lcu_graph_launch(graph_, stream_));
-    } else {
-      enqueue_step(bound);
+    {
+      device_structure_lock lock(device_structure_mutex());  // capture, instantiation, launch: see host_common.hpp
+      if (!graph_ && calls_ >= 2) {
+        LCU_CHECK(lcu_graph_begin_capture(stream_));
+        enqueue_step(bound);
+        LCU_CHECK(lcu_graph_end_capture(stream_, &graph_));
+      }
+      if (graph_) {
+        LCU_CHECK(lcu_graph_launch(graph_, stream_));
+      } else {
+        enqueue_step(bound);
+      }
     }
     std::vector<int> idx(B);
     LCU_CHECK(lcu_d2h(idx.data(), t_argmax_.data(), (size_t)B * sizeof(int), stream_));  // blocks
@@ -125,6 +130,7 @@ struct llama_batch_context_impl final : public llama_batch_context {
  private:
   void drop_graph() {
     if (graph_) {
+      device_structure_lock lock(device_structure_mutex());
       LCU_CHECK(lcu_graph_destroy(graph_));
       graph_ = nullptr;
     }

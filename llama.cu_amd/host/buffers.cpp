@@ -97,6 +97,7 @@ void gpu_buffer_view::copy_to(void* buffer, size_t size) {
 }
 
 gpu_buffer::gpu_buffer(size_t size) {
+  device_structure_lock lock(device_structure_mutex());
   LCU_CHECK(lcu_malloc(&dev_ptr_, size));
   size_ = size;
 }
@@ -107,6 +108,7 @@ gpu_buffer::gpu_buffer(gpu_buffer&& other) : gpu_buffer_view(other.dev_ptr_, oth
 gpu_buffer& gpu_buffer::operator=(gpu_buffer&& other) {
   if (this != &other) {
     if (dev_ptr_) {
+      device_structure_lock lock(device_structure_mutex());
       LCU_CHECK(lcu_free(dev_ptr_));
     }
     dev_ptr_ = std::exchange(other.dev_ptr_, nullptr);
@@ -116,6 +118,7 @@ gpu_buffer& gpu_buffer::operator=(gpu_buffer&& other) {
 }
 gpu_buffer::~gpu_buffer() {
   if (dev_ptr_) {
+    device_structure_lock lock(device_structure_mutex());
     LCU_CHECK(lcu_free(dev_ptr_));
   }
 }

@@ -235,6 +235,7 @@ static bool shapes_supported(llama_params const& p) {
 // ------------------------------------------------------------------------------------------------
 llama_context_impl::llama_context_impl(llama_model* model, int context_len, float temperature)
     : llama_context(static_cast<llama_model_impl*>(model), context_len, temperature) {
+  device_structure_lock lock(device_structure_mutex());
   LCU_CHECK(lcu_init(0));
   LCU_CHECK(lcu_stream_create(&stream_));
   lcu_device_props props;
@@ -254,6 +255,7 @@ llama_context_impl::llama_context_impl(llama_model* model, int context_len, floa
 
 llama_context_impl::~llama_context_impl() {
   lcu_sync(stream_);
+  device_structure_lock lock(device_structure_mutex());
   // Every one-token step has looked at the count of hand-overs that did not arrive before it returned
   // its token (next_token), so there is nothing left to judge here; a context whose steps had to be
   // recomputed says so once more when it goes.
@@ -467,6 +469,7 @@ void llama_context_impl::greedy() {
 
 void llama_context_impl::drop_graph() {
   if (decode_graph_) {
+    device_structure_lock lock(device_structure_mutex());
     LCU_CHECK(lcu_graph_destroy(decode_graph_));
     decode_graph_ = nullptr;
   }
@@ -531,6 +534,7 @@ short llama_context_impl::next_token(std::vector<short> const& new_tokens) {
     // Decode attention has a form for short rows and one for long rows, chosen by the bound it is
     // given; the graph is captured again when the position outgrows the short bound.
     const int bound = (start_pos_ + 1 <= 1024 && context_len_ > 1024) ? 1024 : (int)context_len_;
+    device_structure_lock lock(device_structure_mutex());  // capture, instantiation, launch: see host_common.hpp
     if (decode_graph_ && bound != decode_bound_) {
       LCU_CHECK(lcu_graph_destroy(decode_graph_));
       decode_graph_ = nullptr;

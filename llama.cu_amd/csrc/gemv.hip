@@ -8,7 +8,8 @@
 //     dispatcher balances the many uniform workgroups over the 256 compute units
 //   - each lane issues 16-byte loads (8 halves or 16 codes), U*R of them per batch, requested
 //     before anything else happens in the workgroup (before x is staged or normalised), and the
-//     next batch is requested before the current one is consumed
+//     next batch is requested before the current one is consumed (uint8 rows of up to five
+//     batches: all of them at once, see with_u8_batches)
 //   - each lane loads the pieces of x (or of the norm weights) that match its weights along with
 //     them; when x must be RMS-normalised first, every workgroup requests x before its weights
 //     (loads return in request order), stages it in LDS, reduces the sum of squares there while
@@ -234,8 +235,10 @@ struct batch_t {
 //   void finish(int task, const float (&acc)[R]) const;           epilogue, called by thread 0 only
 // The workgroup's wavefronts take the K chunks of the task's rows round-robin: batch b of
 // wavefront w covers chunks (b * WAVES + w) * U .. + U.  begin() requests the first batch (weights,
-// x, norm weights); the caller may then reduce the norm statistics; run() does the rest and ends
-// with the cross-wavefront sum.
+// x, norm weights), or with NB > 0 all NB batches of the rows; the caller may then reduce the norm
+// statistics; run() does the rest (NB == 0: a loop that requests one batch ahead; NB > 0: the
+// batches summed in the same order, K <= NB * WAVES * U * CHUNK) and ends with the
+// cross-wavefront sum.
 template <bool U8, int R, int U, bool NORM, class Tasks, int NB = 0>
 struct stream_t {
   using batch = batch_t<U8, R, U, NORM>;

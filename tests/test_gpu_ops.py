@@ -134,7 +134,10 @@ def test_gemv_exact_cases(gpu):
     G.release()
 
 
-@pytest.mark.parametrize("K,N", [(4096, 4096), (4096, 11008), (11008, 4096), (256, 40), (1024 + 128, 77), (6656, 17920)])
+# rows of one to six batches of the workgroup (4096 codes each): two to five are requested at once, one
+# and six go through the loop; two and four rows per workgroup (N below / from 6144)
+@pytest.mark.parametrize("K,N", [(4096, 4096), (4096, 11008), (11008, 4096), (256, 40), (1024 + 128, 77), (6656, 17920),
+                                 (17920, 300), (13824, 100), (22016, 64), (8192, 6200), (17920, 6152)])
 def test_gemv_u8(gpu, K, N):
     G = gpu
     x = normal((1, K), 0, 200, 1.0)

@@ -484,7 +484,30 @@ __global__ void embed_kernel(half_t* __restrict__ out, const short* __restrict__
   }
 }
 
-// embed_uint8, llama_cu.cu:46-62
+// embed_uint8, llama_cu.cu:46-62, sixteen codes per thread (one 16-byte request; they share a scale when
+// the block is a multiple of 16): grid (ids, pieces of 4096 codes).  The decode step's single row took
+// 15 us with one element per thread and loop trip.
+__global__ __launch_bounds__(256) void embed_u8x16_kernel(half_t* __restrict__ out, const short* __restrict__ ids,
+                                                          int dim, const uint8_t* __restrict__ codes,
+                                                          const half_t* __restrict__ scales, int block, int n_vocab) {
+  const int i = (blockIdx.y * 256 + threadIdx.x) * 16;
+  if (i >= dim) return;
+  const int id = ids[blockIdx.x];
+  half8_t r[2] = {(half8_t)(0.0f), (half8_t)(0.0f)};
+  if (id >= 0 && id < n_vocab) {
+    const uint4_t q = *reinterpret_cast<const uint4_t*>(codes + (size_t)id * dim + i);
+    const float s = (float)scales[(size_t)id * (dim / block) + i / block];
+#pragma unroll
+    for (int e = 0; e < 16; ++e) {
+      r[e / 8][e % 8] = dequant_one((q[e / 4] >> (8 * (e % 4))) & 0xFF, s);
+    }
+  }
+  half8_t* dst = reinterpret_cast<half8_t*>(out + (size_t)blockIdx.x * dim + i);
+  dst[0] = r[0];
+  dst[1] = r[1];
+}
+
+// any block size and row length: one element per thread and trip
 __global__ void embed_u8_kernel(half_t* __restrict__ out, const short* __restrict__ ids, int dim,
                                 const uint8_t* __restrict__ codes, const half_t* __restrict__ scales, int block,
                                 int n_vocab) {
@@ -879,9 +902,15 @@ int lcu_embed_u8(void* out_dev, const void* ids_dev, int n_ids, int dim, const v
   LCU_REQUIRE(n_ids >= 0 && dim > 0 && block > 0 && dim % block == 0 && n_vocab > 0,
               "lcu_embed_u8: bad shape n %d dim %d block %d", n_ids, dim, block);
   if (n_ids == 0) return LCU_OK;
-  embed_u8_kernel<<<n_ids, 256, 0, as_stream(stream)>>>((half_t*)out_dev, (const short*)ids_dev, dim,
-                                                        (const uint8_t*)codes_dev, (const half_t*)scales_dev, block,
-                                                        n_vocab);
+  if (dim % 16 == 0 && block % 16 == 0) {
+    embed_u8x16_kernel<<<dim3(n_ids, (dim + 4095) / 4096), 256, 0, as_stream(stream)>>>(
+        (half_t*)out_dev, (const short*)ids_dev, dim, (const uint8_t*)codes_dev, (const half_t*)scales_dev, block,
+        n_vocab);
+  } else {
+    embed_u8_kernel<<<n_ids, 256, 0, as_stream(stream)>>>((half_t*)out_dev, (const short*)ids_dev, dim,
+                                                          (const uint8_t*)codes_dev, (const half_t*)scales_dev, block,
+                                                          n_vocab);
+  }
   LCU_LAUNCH_CHECK();
   return LCU_OK;
 }

@@ -501,7 +501,24 @@ def test_embed_bit_exact(gpu):
     bad = np.array([1000, -1], dtype=np.int16)
     G.B.check(G.L().lcu_embed(out_d.ptr, G.dev_keep(bad).ptr, 2, dim, G.dev_keep(table).ptr, vocab, None))
     assert (G.host(out_d, (2, dim)) == 0).all()
+    G.B.check(G.L().lcu_embed_u8(out_d.ptr, G.dev_keep(bad).ptr, 2, dim, G.dev_keep(codes).ptr,
+                                 G.dev_keep(scales).ptr, 128, vocab, None))
+    assert (G.host(out_d, (2, dim)) == 0).all()
     G.release()
+    # uint8 rows of more than one piece of 4096 codes (sixteen codes per thread), and a block size that is
+    # not a multiple of 16 (one code per thread)
+    for vocab, dim, block in ((40, 6656, 128), (40, 4096 + 16, 16), (50, 480, 24)):
+        table = normal((vocab, dim), 0, 901, 0.02)
+        codes, scales = O.quantize_absmax_u8(table, block)
+        ids = np.array([vocab - 1, 0, 7, vocab, 7], dtype=np.int16)
+        out_d = G.empty((len(ids), dim))
+        G.B.check(G.L().lcu_embed_u8(out_d.ptr, G.dev_keep(ids).ptr, len(ids), dim, G.dev_keep(codes).ptr,
+                                     G.dev_keep(scales).ptr, block, vocab, None))
+        got = G.host(out_d, (len(ids), dim))
+        want = O.embed_u8(np.where(ids < vocab, ids, 0).astype(np.int16), codes, scales, block)
+        want[3] = 0
+        assert (got.view(np.uint16) == want.view(np.uint16)).all()
+        G.release()
 
 
 def test_argmax_first_maximum(gpu):

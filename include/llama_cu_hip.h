@@ -141,6 +141,13 @@ int lcu_embed(void* out_dev, const void* ids_dev, int n_ids, int dim, const void
               int n_vocab, void* stream);
 int lcu_embed_u8(void* out_dev, const void* ids_dev, int n_ids, int dim, const void* codes_dev,
                  const void* scales_dev, int block, int n_vocab, void* stream);
+/* embed / embed_uint8 (launch sites 1090, 1094) and the first layer's rms_norm (1129) of the same rows in
+ * one launch: x_out gets the rows, norm_out their norm under weights_dev.  block 0: table_dev is the fp16
+ * table and scales_dev is ignored; else table_dev holds codes (block a multiple of 8 dividing dim).
+ * dim a multiple of 8, at most 8192.  Same values as lcu_embed[_u8] followed by lcu_rmsnorm. */
+int lcu_embed_rmsnorm(void* x_out_dev, void* norm_out_dev, const void* ids_dev, int n_ids, int dim,
+                      const void* table_dev, const void* scales_dev, int block, int n_vocab,
+                      const void* weights_dev, float eps, void* stream);
 /* the host argmax of llama_cu.cu:1205-1209 done on the device: index of the first maximum of n
  * fp16 values compared as float, written as int32 */
 int lcu_argmax_f16(void* out_index_dev, const void* values_dev, int n, void* stream);

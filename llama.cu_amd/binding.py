@@ -60,6 +60,7 @@ SIGNATURES = {
     "lcu_attention_decode_static": (i32, [vp, vp, vp, vp, i32, i32, i32, vp]),
     "lcu_embed": (i32, [vp, vp, i32, i32, vp, i32, vp]),
     "lcu_embed_u8": (i32, [vp, vp, i32, i32, vp, vp, i32, i32, vp]),
+    "lcu_embed_rmsnorm": (i32, [vp, vp, vp, i32, i32, vp, vp, i32, i32, vp, f32, vp]),
     "lcu_argmax_f16": (i32, [vp, vp, i32, vp]),
     "lcu_softmax_argmax": (i32, [vp, vp, vp, i32, f32, vp]),
     "lcu_sample_row": (i32, [vp, vp, i32, u64, vp, vp]),

@@ -523,6 +523,81 @@ __global__ void embed_u8_kernel(half_t* __restrict__ out, const short* __restric
   }
 }
 
+// embed / embed_uint8 followed by rms_norm of the same rows (llama_cu.cu:1087-1097, then 1129 of the
+// first layer) in one launch: a block gathers its row (dequantised where the table is uint8), writes it
+// and normalises it from LDS with rmsnorm_kernel's arithmetic.  The norm weights are requested before the
+// id is known.  cols a multiple of 8, at most 8192; block 0 (fp16 table) or a multiple of 8.
+template <bool U8>
+__global__ __launch_bounds__(256) void embed_rmsnorm_kernel(half_t* __restrict__ x_out, half_t* __restrict__ norm_out,
+                                                            const short* __restrict__ ids, int cols,
+                                                            const void* __restrict__ table,
+                                                            const half_t* __restrict__ scales, int block, int n_vocab,
+                                                            const half_t* __restrict__ weights, float eps) {
+  extern __shared__ half_t xs[];
+  __shared__ __attribute__((aligned(16))) float red[8];
+  constexpr int P = 4;
+  half8_t wp[P];
+#pragma unroll
+  for (int j = 0; j < P; ++j) {
+    const int i = (threadIdx.x + 256 * j) * 8;
+    wp[j] = i < cols ? *reinterpret_cast<const half8_t*>(weights + i) : (half8_t)(0.0f);
+  }
+  const int id = ids[blockIdx.x];
+  const bool ok = id >= 0 && id < n_vocab;
+  half_t* x = x_out + (size_t)blockIdx.x * cols;
+  half_t* y = norm_out + (size_t)blockIdx.x * cols;
+#pragma unroll
+  for (int j = 0; j < P; ++j) {
+    const int i = (threadIdx.x + 256 * j) * 8;
+    if (i >= cols) continue;
+    half8_t v = (half8_t)(0.0f);
+    if (ok) {
+      if constexpr (U8) {
+        const uint2 q = *reinterpret_cast<const uint2*>((const uint8_t*)table + (size_t)id * cols + i);
+        const float sc = (float)scales[(size_t)id * (cols / block) + i / block];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          v[e] = dequant_one(((e < 4 ? q.x : q.y) >> (8 * (e % 4))) & 0xFF, sc);
+        }
+      } else {
+        v = *reinterpret_cast<const half8_t*>((const half_t*)table + (size_t)id * cols + i);
+      }
+    }
+    *reinterpret_cast<half8_t*>(xs + i) = v;
+    *reinterpret_cast<half8_t*>(x + i) = v;
+  }
+  __syncthreads();
+  float s = 0.0f;
+  int i = threadIdx.x;
+  for (; i + 7 * 256 < cols; i += 8 * 256) {
+    float v[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) v[u] = (float)xs[i + u * 256];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) s = fmaf(v[u], v[u], s);
+  }
+  for (; i < cols; i += 256) {
+    float v = (float)xs[i];
+    s = fmaf(v, v, s);
+  }
+  const float total = block256_sum_ref_order_dpp(s, red);
+  const float rms_inv = 1.0f / sqrtf(total / (float)cols + eps);
+#pragma unroll
+  for (int j = 0; j < P; ++j) {
+    const int k = (threadIdx.x + 256 * j) * 8;
+    if (k < cols) {
+      const half8_t xv = *reinterpret_cast<const half8_t*>(xs + k);
+      half8_t r;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const half_t inner = round_f16((float)xv[e] * rms_inv);
+        r[e] = round_f16((float)wp[j][e] * (float)inner);
+      }
+      *reinterpret_cast<half8_t*>(y + k) = r;
+    }
+  }
+}
+
 // exp_ieee on plain fp32 values (a check of the exponential every softmax and SiLU here uses)
 __global__ void exp_kernel(float* __restrict__ out, const float* __restrict__ in, size_t n) {
   const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -910,6 +985,29 @@ int lcu_embed_u8(void* out_dev, const void* ids_dev, int n_ids, int dim, const v
     embed_u8_kernel<<<n_ids, 256, 0, as_stream(stream)>>>((half_t*)out_dev, (const short*)ids_dev, dim,
                                                           (const uint8_t*)codes_dev, (const half_t*)scales_dev, block,
                                                           n_vocab);
+  }
+  LCU_LAUNCH_CHECK();
+  return LCU_OK;
+}
+
+int lcu_embed_rmsnorm(void* x_out_dev, void* norm_out_dev, const void* ids_dev, int n_ids, int dim,
+                      const void* table_dev, const void* scales_dev, int block, int n_vocab, const void* weights_dev,
+                      float eps, void* stream) {
+  LCU_REQUIRE(x_out_dev && norm_out_dev && ids_dev && table_dev && weights_dev, "lcu_embed_rmsnorm: null pointer");
+  LCU_REQUIRE(n_ids >= 0 && dim > 0 && dim % 8 == 0 && dim <= 8192 && n_vocab > 0,
+              "lcu_embed_rmsnorm: bad shape n %d dim %d (dim a multiple of 8, at most 8192)", n_ids, dim);
+  LCU_REQUIRE(block == 0 || (scales_dev && block % 8 == 0 && dim % block == 0),
+              "lcu_embed_rmsnorm: block %d unsupported (0 for an fp16 table, else a multiple of 8 dividing dim, with scales)",
+              block);
+  if (n_ids == 0) return LCU_OK;
+  if (block > 0) {
+    embed_rmsnorm_kernel<true><<<n_ids, 256, (size_t)dim * 2, as_stream(stream)>>>(
+        (half_t*)x_out_dev, (half_t*)norm_out_dev, (const short*)ids_dev, dim, table_dev, (const half_t*)scales_dev, block,
+        n_vocab, (const half_t*)weights_dev, eps);
+  } else {
+    embed_rmsnorm_kernel<false><<<n_ids, 256, (size_t)dim * 2, as_stream(stream)>>>(
+        (half_t*)x_out_dev, (half_t*)norm_out_dev, (const short*)ids_dev, dim, table_dev, nullptr, 0, n_vocab,
+        (const half_t*)weights_dev, eps);
   }
   LCU_LAUNCH_CHECK();
   return LCU_OK;

@@ -343,13 +343,13 @@ void llama_context_impl::matmul_multi(void* const* outs, const void* lhs, weight
 
 // The layer loop for n new rows sitting in t_embed_; positions start_pos_ .. start_pos_ + n - 1.
 // n == 1 takes the fused decode kernels, which read the position from t_step_ on the device.
-void llama_context_impl::enqueue_layers(int n) {
+void llama_context_impl::enqueue_layers(int n, bool first_norm_ready) {
   llama_params const& p = model_->params;
   const int dim = p.dim, ffn = p.ffn_dim(), heads = p.n_heads;
   const int sp = start_pos_, T = sp + n;
   const int block = p.q_type == quantization_type::uint8 ? p.quantization_block_size : 0;
   char* x = (char*)t_embed_.data();
-  bool norm_ready = false;  // t_norm_ already holds this layer's normalised input
+  bool norm_ready = first_norm_ready;  // t_norm_ already holds this layer's normalised input
   for (size_t l = 0; l < model_->layers.size(); ++l) {
     llama_layer const& L = model_->layers[l];
     char* kc = (char*)kv_[l].k.data();
@@ -509,7 +509,16 @@ short llama_context_impl::next_token(std::vector<short> const& new_tokens) {
     LCU_CHECK(lcu_h2d(t_tokens_.data(), new_tokens.data(), n * sizeof(short), stream_));  // 1086
   }
   auto enqueue_all = [&]() {
-    // 1087-1097
+    // 1087-1097; a one-token step gathers the row and normalises it for the first layer (1129) in one launch
+    const bool quantised = model_->tok_embeddings.quantised;
+    if (n == 1 && dim % 8 == 0 && dim <= 8192 && (!quantised || block % 8 == 0) && !model_->layers.empty()) {
+      LCU_CHECK(lcu_embed_rmsnorm(x, t_norm_.data(), ids, 1, dim, model_->tok_embeddings.data.data(),
+                                  quantised ? model_->tok_embeddings.scales.data() : nullptr, quantised ? block : 0, vocab,
+                                  model_->layers[0].attn_norm.data(), model_->params.norm_eps, stream_));
+      enqueue_layers(n, true);
+      enqueue_head(n);
+      return;
+    }
     if (model_->tok_embeddings.quantised) {
       LCU_CHECK(lcu_embed_u8(x, ids, n, dim, model_->tok_embeddings.data.data(), model_->tok_embeddings.scales.data(),
                              block, vocab, stream_));

@@ -76,7 +76,7 @@ struct llama_context_impl final : public llama_context {
  private:
   void matmul(void* out, const void* lhs, weight_tensor const& w, int M, float beta);
   void matmul_multi(void* const* outs, const void* lhs, weight_tensor const* const* ws, int count, int M);
-  void enqueue_layers(int n);
+  void enqueue_layers(int n, bool first_norm_ready = false);
   void enqueue_head(int n);
   void drop_graph();
   std::vector<kv_cache_layer> kv_;

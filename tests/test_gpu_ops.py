@@ -521,6 +521,35 @@ def test_embed_bit_exact(gpu):
         G.release()
 
 
+def test_embed_rmsnorm_equals_embed_then_rmsnorm(gpu):
+    """The one-token step's first launch: the gathered row and its norm, to the bit what lcu_embed[_u8] and
+    lcu_rmsnorm give one after the other (and so what the oracle gives for them)."""
+    G = gpu
+    for vocab, dim, block in ((300, 4096, 0), (300, 4096, 128), (100, 6656, 128), (64, 264, 0), (64, 264, 8), (20, 8192, 64)):
+        table = normal((vocab, dim), 0, 910, 0.02)
+        w = normal((dim,), 0, 911, 1.0)
+        ids = np.array([vocab - 1, 0, 5, vocab, -3, 5], dtype=np.int16)
+        x_d, n_d = G.empty((len(ids), dim)), G.empty((len(ids), dim))
+        safe = np.where((ids >= 0) & (ids < vocab), ids, 0).astype(np.int16)
+        if block:
+            codes, scales = O.quantize_absmax_u8(table, block)
+            G.B.check(G.L().lcu_embed_rmsnorm(x_d.ptr, n_d.ptr, G.dev_keep(ids).ptr, len(ids), dim, G.dev_keep(codes).ptr,
+                                              G.dev_keep(scales).ptr, block, vocab, G.dev_keep(w).ptr, 1e-6, None))
+            rows = O.embed_u8(safe, codes, scales, block)
+        else:
+            G.B.check(G.L().lcu_embed_rmsnorm(x_d.ptr, n_d.ptr, G.dev_keep(ids).ptr, len(ids), dim, G.dev_keep(table).ptr,
+                                              None, 0, vocab, G.dev_keep(w).ptr, 1e-6, None))
+            rows = O.embed(safe, table)
+        rows[3] = 0
+        rows[4] = 0
+        assert (G.host(x_d, (len(ids), dim)).view(np.uint16) == rows.view(np.uint16)).all()
+        assert (G.host(n_d, (len(ids), dim)).view(np.uint16) == O.rms_norm(rows, w, 1e-6).view(np.uint16)).all()
+        G.release()
+    out = G.empty((1, 8200))
+    assert G.L().lcu_embed_rmsnorm(out.ptr, out.ptr, out.ptr, 1, 8200, out.ptr, None, 0, 10, out.ptr, 1e-6, None) != 0
+    G.release()
+
+
 def test_argmax_first_maximum(gpu):
     G = gpu
     out_d = G.empty((1,), np.int32)

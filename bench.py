@@ -35,7 +35,7 @@ HBM_PEAK_GBS = 8000.0      # MI355X HBM3E
 # 256 MiB copy kernel read under the same counters (FETCH_SIZE reads half the bytes here): see
 # profiles/decode_ffn_up_kernel_llama7b_hbm_traffic.txt and decode_u8_kernels_llama30b_counters.txt.
 # Counters are not read in this script.
-MEASURED_TRAFFIC = {"llama7b_fp16": 180637470, "llama30b_u8": 244917605}
+MEASURED_TRAFFIC = {"llama7b_fp16": 180637530, "llama30b_u8": 244906771}
 MFMA_F16_PEAK_TF = 2500.0  # dense fp16
 
 WORKLOADS = {

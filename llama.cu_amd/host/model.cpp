@@ -576,25 +576,25 @@ short llama_context_impl::next_token(std::vector<short> const& new_tokens) {
   // count that has moved means this step's token is not to be trusted.  It is never returned: the
   // context leaves the hand-over launches for good (something else is holding compute units of this
   // device), and the step is computed again by launches that wait for nobody -- the step is a function
-  // of the token, the position and the cache rows below the position, all untouched.
+  // of the token, the position and the cache rows below the position, all untouched.  A call whose
+  // launches hand nothing over (several tokens, or a context already on the plain launches) does not
+  // depend on the count: if it moves there, somebody else is using this stream's workspace, which is
+  // reported and otherwise harmless to the result.
   if (result.timeouts != timeouts_seen_) {
-    fprintf(stderr, "llama_context: %u hand-over(s) between workgroups of a decode launch did not arrive (is other "
-                    "work holding compute units of this device?); the step is recomputed without them\n",
-            result.timeouts - timeouts_seen_);
+    const unsigned moved = result.timeouts - timeouts_seen_;
     timeouts_seen_ = result.timeouts;
-    ++hand_over_fallbacks_;
-    if (!hand_overs_ || n != 1) {
-      // no launch of such a call hands anything over: somebody else is using this stream's workspace
-      fprintf(stderr, "llama_context: the count moved during a call that hands nothing over\n");
-      raise(SIGSEGV);
-    }
-    hand_overs_ = false;
-    drop_graph();
-    enqueue_all();
-    LCU_CHECK(lcu_d2h(&result, t_argmax_.data(), sizeof(result), stream_));
-    if (result.timeouts != timeouts_seen_) {
-      fprintf(stderr, "llama_context: the recomputed step reports hand-overs as well\n");
-      raise(SIGSEGV);
+    if (hand_overs_ && n == 1) {
+      fprintf(stderr, "llama_context: %u hand-over(s) between workgroups of a decode launch did not arrive (is other "
+                      "work holding compute units of this device?); the step is recomputed without them\n", moved);
+      ++hand_over_fallbacks_;
+      hand_overs_ = false;
+      drop_graph();
+      enqueue_all();
+      LCU_CHECK(lcu_d2h(&result, t_argmax_.data(), sizeof(result), stream_));
+      timeouts_seen_ = result.timeouts;
+    } else {
+      fprintf(stderr, "llama_context: the stream's count of failed hand-overs moved by %u during a call that hands "
+                      "nothing over (is the stream's workspace shared?); the call's result does not depend on it\n", moved);
     }
   }
   start_pos_ += n;

@@ -6,8 +6,8 @@ import sys
 PKG = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(PKG)
 LIB = os.path.join(PKG, "libllama_cu_amd.so")
-# diagnostic build: the same library with the phase timeline of the fused decode launch compiled in
-# (csrc/attention.hip, -DLCU_PHASE_TIMELINE), read by timeline.py
+# diagnostic build: the same library with the phase timelines of the fused decode launch and of the
+# W2 + norm launch compiled in (csrc/attention.hip, csrc/gemv.hip, -DLCU_PHASE_TIMELINE), read by timeline.py
 TIMELINE_LIB = os.path.join(PKG, "libllama_cu_amd_timeline.so")
 
 HIP_SOURCES = ["csrc/runtime.hip", "csrc/elementwise.hip", "csrc/gemv.hip", "csrc/gemm.hip", "csrc/attention.hip"]
@@ -58,12 +58,15 @@ def build(verbose=False):
 
 
 def build_timeline():
-    """libllama_cu_amd_timeline.so: attention.hip recompiled with -DLCU_PHASE_TIMELINE, every other
-    object taken from the last ordinary build (build() first)."""
-    obj = os.path.join(PKG, "build", "attention.hip.timeline.o")
-    subprocess.check_call(["hipcc"] + COMMON + DEVICE + ["-DLCU_PHASE_TIMELINE", "-c", os.path.join(PKG, "csrc/attention.hip"),
-                           "-o", obj], stderr=subprocess.DEVNULL)
-    objs = [obj if os.path.basename(src) == "attention.hip" else os.path.join(PKG, "build", os.path.basename(src) + ".o")
+    """libllama_cu_amd_timeline.so: attention.hip and gemv.hip recompiled with -DLCU_PHASE_TIMELINE, every
+    other object taken from the last ordinary build (build() first)."""
+    instrumented = {}
+    for name in ("attention.hip", "gemv.hip"):
+        obj = os.path.join(PKG, "build", name + ".timeline.o")
+        subprocess.check_call(["hipcc"] + COMMON + DEVICE + ["-DLCU_PHASE_TIMELINE", "-c", os.path.join(PKG, "csrc", name),
+                               "-o", obj], stderr=subprocess.DEVNULL)
+        instrumented[name] = obj
+    objs = [instrumented.get(os.path.basename(src), os.path.join(PKG, "build", os.path.basename(src) + ".o"))
             for src in HIP_SOURCES + HOST_SOURCES]
     subprocess.check_call(["hipcc", "--offload-arch=gfx950", "-shared", "-o", TIMELINE_LIB] + objs)
     return TIMELINE_LIB

@@ -555,6 +555,26 @@ __global__ __launch_bounds__(GEMV_THREADS) void decode_ffn_up_kernel(
 // left there: step counter << 10 | salt), then writes the row and its norm (rmsnorm_kernel's
 // arithmetic).  It is resident while the last GEMV workgroups run, so the norm costs the hand-over
 // and its own arithmetic instead of a launch; its wait is bounded and counts itself when it runs out.
+// Diagnostic builds only (-DLCU_PHASE_TIMELINE): thread 0 of every workgroup of the launch notes the
+// 100 MHz real-time counter when it starts, when its first batch has been summed, and when its result
+// is stored (the follower: start, every word in LDS, norm written, and the sum of squares known); one row per launch (by salt) and
+// workgroup, copied out by lcu_debug_timeline_read_proj.  Nothing of this exists in the ordinary build.
+#ifdef LCU_PHASE_TIMELINE
+constexpr int PTL_POINTS = 4, PTL_LAUNCHES = 64, PTL_GROUPS = 4096;
+static __device__ uint64_t proj_timeline[PTL_LAUNCHES * PTL_GROUPS * PTL_POINTS];
+#define PTL_MARK(point)                                                                                          \
+  do {                                                                                                           \
+    if (threadIdx.x == 0 && blockIdx.x < PTL_GROUPS) {                                                           \
+      proj_timeline[((ptl_launch & (PTL_LAUNCHES - 1)) * PTL_GROUPS + blockIdx.x) * PTL_POINTS + (point)] =      \
+          __builtin_amdgcn_s_memrealtime();                                                                      \
+    }                                                                                                            \
+  } while (0)
+#else
+#define PTL_MARK(point) \
+  do {                  \
+  } while (0)
+#endif
+
 constexpr int FOLLOW_SPIN_LIMIT = 1 << 16;
 constexpr int FOLLOW_PIECES = 8;  // 16-byte requests per thread: N <= 8192
 
@@ -567,6 +587,10 @@ __global__ __launch_bounds__(GEMV_THREADS) void decode_proj_norm_kernel(
   extern __shared__ half_t xs[];  // N halves: the follower's copy of the row
   __shared__ __attribute__((aligned(16))) float red[8];
   __shared__ float part[GEMV_WAVES * R];
+#ifdef LCU_PHASE_TIMELINE
+  const uint32_t ptl_launch = epoch >> 1;  // the salt of a W2 launch is 2 * layer + 1
+#endif
+  PTL_MARK(0);
   epoch = (epoch | (*seq_dev << 10)) & 0x7fffffffu;
   const int n_tasks = (N + R - 1) / R;
   if ((int)blockIdx.x < n_tasks) {
@@ -574,6 +598,7 @@ __global__ __launch_bounds__(GEMV_THREADS) void decode_proj_norm_kernel(
     stream_t<U8, R, U, false, proj_norm_tasks<U8, R>, NB> st(tk, lhs, nullptr, K, block, blockIdx.x);
     st.begin();
     st.run(xs, 1.0f, part);
+    PTL_MARK(2);
     return;
   }
   const int tid = threadIdx.x;
@@ -584,43 +609,48 @@ __global__ __launch_bounds__(GEMV_THREADS) void decode_proj_norm_kernel(
     const int i = (tid + GEMV_THREADS * j) * 8;
     nwp[j] = i < N ? *reinterpret_cast<const half8_t*>(norm_w + i) : (half8_t)(0.0f);
   }
-  // two neighbouring words per request, four requests per statement; a piece past the row reads the
-  // row's first words instead and is ignored
-  uint4_t raw[FOLLOW_PIECES];
+  // two neighbouring words per request, four requests per statement, and one such group of four at a
+  // time (asked for until it is fresh, then put into LDS: sixteen registers for the words instead of
+  // thirty-two, which keeps the whole kernel at the GEMV workgroups' register count and so at eight
+  // workgroups per compute unit; with 80 registers a quarter of the 2048 workgroups of W2 started
+  // only when others had finished).  A piece past the row reads the row's first words instead and
+  // is ignored.  The waits of a wavefront share one budget of polls.
   int spins = 0;
-  while (true) {
-    bool stale = false;
+  bool gave_up = false;
 #pragma unroll
-    for (int j = 0; j < FOLLOW_PIECES; j += 4) {
-      if (GEMV_THREADS * j * 2 >= N / 2) continue;  // the whole group lies past the row (the same for every thread)
-      uint4_t four[4];
-      const int w0 = (tid + GEMV_THREADS * j) * 2, w1 = w0 + GEMV_THREADS * 2, w2 = w1 + GEMV_THREADS * 2,
-                w3 = w2 + GEMV_THREADS * 2;
+  for (int j = 0; j < FOLLOW_PIECES; j += 4) {
+    if (GEMV_THREADS * j * 2 >= N / 2) continue;  // the whole group lies past the row (the same for every thread)
+    uint4_t four[4];
+    const int w0 = (tid + GEMV_THREADS * j) * 2, w1 = w0 + GEMV_THREADS * 2, w2 = w1 + GEMV_THREADS * 2,
+              w3 = w2 + GEMV_THREADS * 2;
+    const int wi[4] = {w0, w1, w2, w3};
+    while (true) {
       load_word_pairs_device_scope(four, words + (w0 < N / 2 ? w0 : 0), words + (w1 < N / 2 ? w1 : 0),
                                    words + (w2 < N / 2 ? w2 : 0), words + (w3 < N / 2 ? w3 : 0));
+      bool stale = false;
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
-        raw[j + e] = four[e];
-        if ((tid + GEMV_THREADS * (j + e)) * 2 < N / 2) stale |= four[e][1] != epoch || four[e][3] != epoch;
+        if (wi[e] < N / 2) stale |= four[e][1] != epoch || four[e][3] != epoch;
       }
+      if (__builtin_amdgcn_ballot_w64(stale) == 0 || gave_up) break;
+      if (++spins > FOLLOW_SPIN_LIMIT) {
+        if ((tid & 63) == 0) atomicAdd(timeouts, 1u);
+        gave_up = true;
+        break;
+      }
+      __builtin_amdgcn_s_sleep(2);
     }
-    if (__builtin_amdgcn_ballot_w64(stale) == 0) break;
-    if (++spins > FOLLOW_SPIN_LIMIT) {
-      if ((tid & 63) == 0) atomicAdd(timeouts, 1u);
-      break;
-    }
-    __builtin_amdgcn_s_sleep(2);
-  }
 #pragma unroll
-  for (int j = 0; j < FOLLOW_PIECES; ++j) {
-    const int w0 = (tid + GEMV_THREADS * j) * 2;
-    if (w0 < N / 2) {
-      uint32_t* dst = reinterpret_cast<uint32_t*>(xs + 2 * w0);
-      dst[0] = raw[j][0];
-      dst[1] = raw[j][2];
+    for (int e = 0; e < 4; ++e) {
+      if (wi[e] < N / 2) {
+        uint32_t* dst = reinterpret_cast<uint32_t*>(xs + 2 * wi[e]);
+        dst[0] = four[e][0];
+        dst[1] = four[e][2];
+      }
     }
   }
   __syncthreads();
+  PTL_MARK(1);
   // rms_norm, llama_cu.cu:66-107, as rmsnorm_kernel: thread t owns elements t, t + 256, ...
   float s = 0.0f;
   {
@@ -640,6 +670,7 @@ __global__ __launch_bounds__(GEMV_THREADS) void decode_proj_norm_kernel(
   }
   const float total = block256_sum_ref_order_dpp(s, red);
   const float rms_inv = 1.0f / sqrtf(total / (float)N + eps);
+  PTL_MARK(3);
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
     const int i = (tid + GEMV_THREADS * j) * 8;
@@ -655,6 +686,7 @@ __global__ __launch_bounds__(GEMV_THREADS) void decode_proj_norm_kernel(
     *reinterpret_cast<half8_t*>(x_io + i) = xv;
     *reinterpret_cast<half8_t*>(norm_out + i) = r;
   }
+  PTL_MARK(2);
 }
 
 // calls f with the number of 16-byte pieces of x per thread (x_stage_t) that covers dim <= 24576
@@ -915,5 +947,23 @@ int lcu_decode_logits(void* logits_dev, const void* x_dev, const void* norm_w_de
   LCU_LAUNCH_CHECK();
   return LCU_OK;
 }
+
+#ifdef LCU_PHASE_TIMELINE
+// diagnostic builds only: clears (out_host == NULL) or copies out the timeline of the W2 launches of
+// lcu_decode_proj_norm (odd salts), uint64[64 launches][4096 workgroups][4 points] of the 100 MHz counter
+int lcu_debug_timeline_read_proj(void* out_host, size_t bytes) {
+  void* dev = nullptr;
+  LCU_HIP(hipGetSymbolAddress(&dev, HIP_SYMBOL(proj_timeline)));
+  LCU_HIP(hipDeviceSynchronize());
+  if (out_host == nullptr) {
+    LCU_HIP(hipMemset(dev, 0, sizeof(uint64_t) * PTL_LAUNCHES * PTL_GROUPS * PTL_POINTS));
+  } else {
+    LCU_REQUIRE(bytes <= sizeof(uint64_t) * PTL_LAUNCHES * PTL_GROUPS * PTL_POINTS,
+                "lcu_debug_timeline_read_proj: too many bytes");
+    LCU_HIP(hipMemcpy(out_host, dev, bytes, hipMemcpyDeviceToHost));
+  }
+  return LCU_OK;
+}
+#endif
 
 }  // extern "C"
